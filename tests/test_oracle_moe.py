@@ -1,0 +1,101 @@
+"""Pins for oracle/moe.py, oracle/routing.py and oracle/metrics.py: an independent dense
+formulation, hand-computable special cases, closed forms."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import mxfp4, moe, routing, metrics
+
+
+def _layer(rng, E, T, k, H, I):
+    hidden = mxfp4.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    w1 = (rng.standard_normal((E, 2 * I, H)) * 0.02).astype(np.float32)
+    w2 = (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32)
+    w1q, w1s = mxfp4.quantize_mxfp4(w1)
+    w2q, w2s = mxfp4.quantize_mxfp4(w2)
+    tw, ti = routing.softmax_topk(rng.standard_normal((T, E)), k)
+    return hidden, w1q, w1s, w2q, w2s, tw, ti
+
+
+@pytest.mark.parametrize("act", ["a4", "a16"])
+def test_against_dense_formulation(act):
+    rng = np.random.default_rng(0)
+    E, T, k, H, I = 4, 9, 2, 64, 32
+    hidden, w1q, w1s, w2q, w2s, tw, ti = _layer(rng, E, T, k, H, I)
+    out, a2, per_slot = moe.moe_ref(hidden, w1q, w1s, w2q, w2s, tw, ti, act=act, return_parts=True)
+    # independent: every token through every expert in float64, combined with a dense routing matrix
+    W1 = mxfp4.dequantize_mxfp4(w1q, w1s).astype(np.float64)
+    W2 = mxfp4.dequantize_mxfp4(w2q, w2s).astype(np.float64)
+    qd = (lambda v: mxfp4.dequantize_mxfp4(*mxfp4.quantize_mxfp4(v.astype(np.float32))).astype(np.float64)) \
+        if act == "a4" else (lambda v: v.astype(np.float64))
+    x = qd(hidden)
+    gu = np.einsum("th,enh->etn", x, W1)
+    g, u = gu[..., :I], gu[..., I:]
+    a = mxfp4.bf16_round((g / (1 + np.exp(-g)) * u).astype(np.float32))
+    y = np.einsum("eti,ehi->eth", qd(a.reshape(E * T, I)).reshape(E, T, I), W2)
+    dense = np.zeros((T, H))
+    for t in range(T):
+        for s in range(k):
+            dense[t] += mxfp4.bf16_round((y[ti[t, s], t] * tw[t, s]).astype(np.float32))
+    # float64 vs float32 matmul can flip single bf16 / e2m1 roundings; the bulk must agree tightly
+    assert metrics.cosine(out, dense) > 0.99999
+    assert np.median(np.abs(out - dense)) < 1e-3 * np.sqrt(np.mean(dense ** 2))
+    assert a2.shape == (T, k, I) and per_slot.shape == (T, k, H)
+
+
+def test_single_expert_identity_weights():
+    # one expert, w1 = [4*I_H ; 4*I_H] (gate = up = 4x), w2 = identity -> out = silu(4x) * 4x * weight
+    H = I = 32
+    eye = np.eye(H, dtype=np.float32)
+    w1q, w1s = mxfp4.quantize_mxfp4(np.concatenate([4 * eye, 4 * eye])[None])
+    w2q, w2s = mxfp4.quantize_mxfp4(eye[None])
+    assert (mxfp4.dequantize_mxfp4(w1q, w1s)[0, :H] == 4 * eye).all()
+    x = mxfp4.bf16_round(np.linspace(-1, 1, 3 * H, dtype=np.float32).reshape(3, H))
+    tw = np.array([[1.0], [0.5], [0.0]], dtype=np.float32)
+    ti = np.zeros((3, 1), dtype=np.int32)
+    out = moe.moe_ref(x, w1q, w1s, w2q, w2s, tw, ti, act="a16")
+    g = 4 * x
+    expect = mxfp4.bf16_round(mxfp4.bf16_round(g / (1 + np.exp(-g)) * g) * tw)
+    np.testing.assert_allclose(out, expect, rtol=2 ** -7, atol=1e-6)
+    assert (out[2] == 0).all()
+
+
+def test_bias_and_expert_subset():
+    rng = np.random.default_rng(1)
+    E, T, k, H, I = 4, 6, 2, 64, 32
+    hidden, w1q, w1s, w2q, w2s, tw, ti = _layer(rng, E, T, k, H, I)
+    b1 = (rng.standard_normal((E, 2 * I)) * 0.01).astype(np.float32)
+    b2 = (rng.standard_normal((E, H)) * 0.01).astype(np.float32)
+    full = moe.moe_ref(hidden, w1q, w1s, w2q, w2s, tw, ti, bias1=b1, bias2=b2)
+    parts = sum(moe.moe_ref(hidden, w1q, w1s, w2q, w2s, tw, ti, bias1=b1, bias2=b2, experts=[e]) for e in range(E))
+    np.testing.assert_allclose(full, parts, rtol=1e-6, atol=1e-7)
+    nob = moe.moe_ref(hidden, w1q, w1s, w2q, w2s, tw, ti)
+    assert np.abs(full - nob).max() > 0
+
+
+def test_routers():
+    rng = np.random.default_rng(2)
+    logits = rng.standard_normal((50, 64))
+    w, ids = routing.softmax_topk(logits, 4)
+    assert np.allclose(w.sum(1), 1, atol=1e-6) and all(len(set(r)) == 4 for r in ids.tolist())
+    assert (ids[:, 0] == logits.argmax(1)).all()
+    w, ids = routing.grouped_sigmoid_topk(logits, 8, n_group=8, topk_group=4)
+    assert np.allclose(w.sum(1), 1, atol=1e-6)
+    for t in range(50):
+        assert len(set(ids[t].tolist())) == 8
+        assert len(set((ids[t] // 8).tolist())) <= 4
+        # brute force: best 4 groups by the sum of their two best sigmoids, then best 8 inside
+        s = 1 / (1 + np.exp(-logits[t]))
+        gs = [np.sort(s[g * 8:(g + 1) * 8])[-2:].sum() for g in range(8)]
+        groups = sorted(range(8), key=lambda g: -gs[g])[:4]
+        cand = sorted([e for g in groups for e in range(g * 8, g * 8 + 8)], key=lambda e: -s[e])[:8]
+        assert sorted(cand) == sorted(ids[t].tolist())
+
+
+def test_metrics_closed_forms():
+    x = np.arange(1, 9, dtype=np.float32)
+    assert metrics.calc_diff(x, x) == 0 and abs(metrics.calc_diff(x, -x) - 2) < 1e-12
+    assert abs(metrics.calc_diff(x, 0 * x) - 1) < 1e-12
+    assert abs(metrics.calc_diff(x, 3 * x) - (1 - 6 / 10)) < 1e-12      # 1 - 2c/(1+c^2)
+    assert abs(metrics.cosine(x, 5 * x) - 1) < 1e-12
+    assert abs(metrics.max_err_over_rms(x + 0.5, x) - 0.5 / np.sqrt(np.mean(x.astype(np.float64) ** 2))) < 1e-12
