@@ -1,0 +1,105 @@
+/* C ABI of libpyhip_moe.so: MXFP4 fused-MoE for MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HIP device memory of the
+ * current device; `stream` is a hipStream_t (NULL = default stream).  All calls only enqueue
+ * work; none synchronises.  Return value: 0 = ok, 1 = invalid argument, 2 = HIP error; the
+ * message of the last failure on the calling thread is returned by pyhip_moe_last_error().
+ *
+ * Each entry point names the reference interface (tingqli/pyhip, file:line) whose job it does.
+ */
+#ifndef PYHIP_MOE_H
+#define PYHIP_MOE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* pyhip_stream_t; /* hipStream_t */
+
+/* ABI revision of this header. */
+int pyhip_moe_abi_version(void);
+
+/* Message of the last failed call on this thread (replaces the Python exception text of
+ * hip_check_error, src/core/hiptools.py:37-39). */
+const char* pyhip_moe_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Routing sort.  Replaces aiter.fused_moe.moe_sorting as called at src/contrib/fused_moe.py:283,
+ * 301-305,368-372 (CPU statement of the result: src/contrib/fused_moe.py:56-100; in-tree C++
+ * statement: archive/ck_tile/ck_tile/host/reference/reference_moe_sorting.hpp:13-117) and the
+ * JIT sorter src/contrib/moe_sorting.py:7-212.
+ *
+ *   n_blk             = pyhip_moe_sorting_max_blocks(tokens, topk, experts, block_size)
+ *   sorted_ids        u32 [n_blk * block_size]  (slot << 24) | token ; padding (topk << 24) | tokens
+ *   sorted_weights    f32 [n_blk * block_size]  routing weight ; padding 0
+ *   sorted_expert_ids u32 [n_blk]               (local) expert of each block ; 0xFFFFFFFF past the end
+ *   num_valid_ids     u32 [2]                   { padded total, number of (local) tokens }
+ * Order: experts ascending, then tokens, then slots (deterministic).  expert_mask (device int32
+ * [experts], may be NULL) drops the pairs of masked experts and makes expert ids local;
+ * num_local_tokens (device int32 scalar, may be NULL) limits the tokens that are read.
+ * moe_out (may be NULL) is zero-filled over moe_out_bytes, as the reference's sorter does for the
+ * layer output.  workspace: pyhip_moe_sorting_workspace_bytes() bytes of device memory. */
+int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size);
+int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, int experts);
+int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk, int experts,
+                      int block_size, const int32_t* expert_mask, const int32_t* num_local_tokens,
+                      uint32_t* sorted_ids, float* sorted_weights, uint32_t* sorted_expert_ids,
+                      uint32_t* num_valid_ids, void* moe_out, int64_t moe_out_bytes, void* workspace,
+                      int64_t workspace_bytes, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dynamic MXFP4 quantisation of bf16 activations (1x32 blocks, e8m0 scale
+ * 2^(floor(log2 amax) - 2), e2m1 round-to-nearest-even).  Replaces
+ * aiter.get_hip_quant(QuantType.per_1x32) + fp4_utils.moe_mxfp4_sort as used at
+ * tests/contrib/moe/test_moe.py:664-679,732-744.
+ *   x       bf16 [rows, K], row stride row_stride_elems
+ *   q       u8   [rows, K/2]   low nibble = even element
+ *   scales  u8   [rows, pyhip_moe_act_scale_stride(K)]  every 16-byte group stored 4x4-transposed:
+ *           byte kb*4 + i = scale of block 4*i + kb (the grouped GEMM's operand order)
+ *   rows_limit  device u32 scalar (may be NULL): only rows < *rows_limit are processed. */
+int64_t pyhip_moe_act_scale_stride(int K);
+int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K, uint8_t* q,
+                              uint8_t* scales, const uint32_t* rows_limit, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Stage 1: gate_up grouped GEMM with fused SiLU(gate)*up.  Replaces moe_gemm_mxfp4(gate_up=True),
+ * src/contrib/moe_gemm_mxfp4.py:972-1290 (launch: tests/contrib/moe/test_moe.py:720-730).
+ *   a_q/a_scale  quantised hidden states [tokens, hidden/2] / scales (token order, see above)
+ *   w1           u8 [experts, 2*inter, hidden/2], gate rows then up rows, pre-shuffled as
+ *                src/misc.py:116-130 (pre_shuffle(x, 16))
+ *   w1_scale     e8m0, shuffled as tests/contrib/moe/test_fused_moe.py:222-236 over [experts*2*inter, hidden/32]
+ *   bias1        bf16 [experts, 2*inter] or NULL
+ *   a2           bf16 [n_blk*block_m, inter], row = sorted position (padding rows are zero)
+ * block_m must equal the block_size the sort ran with; hidden % 512 == 0, inter % 128 == 0. */
+int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
+                          const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
+                          const uint32_t* num_valid_ids, void* a2_bf16, int tokens, int topk, int experts,
+                          int hidden, int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
+
+/* Stage 2: down grouped GEMM, times the routing weight.  Replaces moe_gemm_mxfp4(gate_up=False),
+ * src/contrib/moe_gemm_mxfp4.py:1291-1333 (launch: tests/contrib/moe/test_moe.py:751-763).
+ *   a2_q/a2_scale  quantised stage-1 output [n_blk*block_m, inter/2] / scales (sorted-row order)
+ *   w2, w2_scale   u8 [experts, hidden, inter/2] pre-shuffled; e8m0 shuffled over [experts*hidden, inter/32]
+ *   bias2          bf16 [experts, hidden] or NULL (added before the routing weight)
+ *   out3           bf16 [tokens, topk, hidden]; only (token, slot) pairs that were sorted are written
+ * inter % 512 == 0, hidden % 256 == 0. */
+int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                          const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
+                          const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* out3_bf16,
+                          int tokens, int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
+                          pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.
+ * Replaces moe_gemm_final_reduce_bf16, src/contrib/moe_gemm_mxfp4.py:199-282
+ * (launch: tests/contrib/moe/test_moe.py:764-771).  out is bf16 or (out_is_f32 != 0) fp32.
+ * num_valid_ids (may be NULL): when given, only tokens < num_valid_ids[1] are reduced. */
+int pyhip_moe_topk_reduce(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden, int out_is_f32,
+                          const uint32_t* num_valid_ids, pyhip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PYHIP_MOE_H */

@@ -1,0 +1,71 @@
+// Shared device/host helpers for the MXFP4 fused-MoE kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <utility>
+#include <type_traits>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned int u32;
+typedef unsigned long long u64;
+
+#define PYHIP_OK 0
+#define PYHIP_ERR_INVALID 1   // argument check failed (message in pyhip_moe_last_error)
+#define PYHIP_ERR_HIP 2       // a HIP runtime call failed (message in pyhip_moe_last_error)
+
+#define WAVE 64
+
+// error plumbing shared by every translation unit of the library (defined in capi.hip)
+extern "C" void pyhip_set_error(const char* fmt, ...);
+
+#define PYHIP_REQUIRE(cond, ...)                 \
+    do {                                         \
+        if(!(cond)) {                            \
+            pyhip_set_error(__VA_ARGS__);        \
+            return PYHIP_ERR_INVALID;            \
+        }                                        \
+    } while(0)
+
+#define PYHIP_CHECK_LAUNCH(name)                                                  \
+    do {                                                                          \
+        hipError_t e_ = hipGetLastError();                                        \
+        if(e_ != hipSuccess) {                                                    \
+            pyhip_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+            return PYHIP_ERR_HIP;                                                 \
+        }                                                                         \
+    } while(0)
+
+__device__ __forceinline__ u32 pack_bf16x2(float a, float b)
+{
+    v2f v = {a, b};
+    v2bf r = __builtin_convertvector(v, v2bf);   // v_cvt_pk_bf16_f32: round to nearest even
+    return __builtin_bit_cast(u32, r);
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(u32 hi16) { return __builtin_bit_cast(float, hi16 << 16); }
+
+// silu(x) = x / (1 + 2^(-x*log2 e)) with the hardware exp2 / rcp approximations
+__device__ __forceinline__ float silu_f32(float x)
+{
+    float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+// compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>)
+{
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}

@@ -1,0 +1,69 @@
+// Top-k reduction of the down-projection output: out[t, :] = sum over slots of in[t, slot, :],
+// slots added in index order in fp32, one rounding to the output type at the end
+// (what the reference's moe_gemm_final_reduce_bf16 computes, src/contrib/moe_gemm_mxfp4.py:199-282).
+#include "common.h"
+
+template <bool OUT_F32>
+__global__ void __launch_bounds__(256)
+    moe_topk_reduce_kernel(const uint4* __restrict__ in, void* __restrict__ out, long long T, int k, int H8,
+                           const u32* __restrict__ tokens_limit)
+{
+    if(tokens_limit)
+    {
+        long long lim = (long long)tokens_limit[1];
+        T             = T < lim ? T : lim;
+    }
+    const long long total = T * H8;
+    for(long long id = (long long)blockIdx.x * 256 + threadIdx.x; id < total; id += (long long)gridDim.x * 256)
+    {
+        const long long t = id / H8;
+        const int c       = (int)(id - t * H8);
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        const uint4* p = in + (t * k) * H8 + c;
+        for(int s = 0; s < k; s++)
+        {
+            uint4 v = p[(long long)s * H8];
+            acc[0] += bf16_bits_to_f32(v.x & 0xFFFFu); acc[1] += bf16_bits_to_f32(v.x >> 16);
+            acc[2] += bf16_bits_to_f32(v.y & 0xFFFFu); acc[3] += bf16_bits_to_f32(v.y >> 16);
+            acc[4] += bf16_bits_to_f32(v.z & 0xFFFFu); acc[5] += bf16_bits_to_f32(v.z >> 16);
+            acc[6] += bf16_bits_to_f32(v.w & 0xFFFFu); acc[7] += bf16_bits_to_f32(v.w >> 16);
+        }
+        if(OUT_F32)
+        {
+            float4* o = (float4*)out + id * 2;
+            o[0]      = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            o[1]      = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+        else
+        {
+            uint4 o;
+            o.x = pack_bf16x2(acc[0], acc[1]);
+            o.y = pack_bf16x2(acc[2], acc[3]);
+            o.z = pack_bf16x2(acc[4], acc[5]);
+            o.w = pack_bf16x2(acc[6], acc[7]);
+            ((uint4*)out)[id] = o;
+        }
+    }
+}
+
+extern "C" int pyhip_moe_topk_reduce(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden,
+                                     int out_is_f32, const uint32_t* num_valid_ids, hipStream_t stream)
+{
+    PYHIP_REQUIRE(in_bf16 && out, "topk_reduce: null pointer");
+    PYHIP_REQUIRE(hidden > 0 && hidden % 8 == 0, "topk_reduce: hidden=%d must be a multiple of 8", hidden);
+    PYHIP_REQUIRE(topk >= 1, "topk_reduce: topk=%d", topk);
+    PYHIP_REQUIRE(((uintptr_t)in_bf16 % 16) == 0 && ((uintptr_t)out % 16) == 0, "topk_reduce: unaligned pointer");
+    if(tokens <= 0)
+        return PYHIP_OK;
+    long long total = (long long)tokens * (hidden / 8);
+    long long grid  = (total + 255) / 256;
+    grid            = grid > 8192 ? 8192 : grid;
+    if(out_is_f32)
+        hipLaunchKernelGGL(moe_topk_reduce_kernel<true>, dim3((unsigned)grid), dim3(256), 0, stream,
+                           (const uint4*)in_bf16, out, (long long)tokens, topk, hidden / 8, num_valid_ids);
+    else
+        hipLaunchKernelGGL(moe_topk_reduce_kernel<false>, dim3((unsigned)grid), dim3(256), 0, stream,
+                           (const uint4*)in_bf16, out, (long long)tokens, topk, hidden / 8, num_valid_ids);
+    PYHIP_CHECK_LAUNCH("moe_topk_reduce_kernel");
+    return PYHIP_OK;
+}

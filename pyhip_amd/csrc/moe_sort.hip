@@ -1,0 +1,424 @@
+// Token routing sort: group (token, slot) pairs by expert, keep (token, slot) order inside an
+// expert, pad every expert's run to the block size.
+//
+// Output contract (what the reference's callers read, src/contrib/fused_moe.py:56-100 and
+// archive/ck_tile/ck_tile/host/reference/reference_moe_sorting.hpp:13-117):
+//   sorted_ids[p]        = (slot << 24) | token, padding = (topk << 24) | num_tokens
+//   sorted_weights[p]    = routing weight, padding = 0
+//   sorted_expert_ids[b] = (local) expert of block b; 0xFFFFFFFF past the last valid block
+//   num_valid_ids        = { padded total, number of (local) tokens }
+// The order is deterministic (no atomics decide a position): a pair's position is
+//   expert_offset[e] + (#pairs of e in earlier workgroups) + (#pairs of e in earlier waves of this
+//   workgroup) + (#pairs of e earlier in this wave's chunk).
+//
+// Three launches for large inputs (histogram -> scan -> scatter) and one single-workgroup
+// launch for decode-sized inputs.
+#include "common.h"
+
+#define SORT_THREADS 256
+#define SORT_WAVES (SORT_THREADS / WAVE)
+#define SMALL_THREADS 1024
+#define SMALL_WAVES (SMALL_THREADS / WAVE)
+#define EXPERT_FILL 0xFFFFFFFFu
+
+struct SortArgs
+{
+    const int* topk_ids;       // [T_all, k]
+    const float* topk_w;       // [T_all, k]
+    const int* expert_mask;    // [E] or null
+    const int* num_local_tok;  // device scalar or null
+    u32* sorted_ids;
+    float* sorted_w;
+    u32* sorted_e;
+    u32* num_valid;
+    u32* ws;                   // workspace: hist[G][E], then per-expert offset[E], total[E], local_id[E]
+    int T_all, k, E, Bm, n_blk, G;
+};
+
+__device__ __forceinline__ int sort_tokens(const SortArgs& a)
+{
+    int T = a.T_all;
+    if(a.num_local_tok)
+    {
+        int t = *a.num_local_tok;
+        T     = t < 0 ? 0 : (t < T ? t : T);
+    }
+    return T;
+}
+
+// pairs handled by one wave: a multiple of 64 so that waves never share a 64-pair group
+__device__ __forceinline__ int wave_chunk(int pairs, int total_waves)
+{
+    int c = (pairs + total_waves - 1) / total_waves;
+    return (c + WAVE - 1) / WAVE * WAVE;
+}
+
+// histogram of the pairs [beg, end) into h[E] (LDS), counting only kept experts
+__device__ __forceinline__ void wave_hist(const SortArgs& a, u32* h, int beg, int end)
+{
+    for(int i = beg + lane_id(); i < end; i += WAVE)
+    {
+        int e = a.topk_ids[i];
+        if(e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0))
+            atomicAdd(&h[e], 1u);
+    }
+}
+
+// writes the pairs [beg, end) to their final positions; base[e] (LDS, private to this wave) is the
+// position of the wave's first pair of expert e and is advanced as groups are consumed
+__device__ __forceinline__ void wave_scatter(const SortArgs& a, u32* base, int beg, int end)
+{
+    const int lane  = lane_id();
+    const u64 lt    = (1ull << lane) - 1ull;
+    for(int g = beg; g < end; g += WAVE)
+    {
+        int i     = g + lane;
+        int e     = -1;
+        float w   = 0.f;
+        if(i < end)
+        {
+            e = a.topk_ids[i];
+            w = a.topk_w[i];
+        }
+        bool keep = e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
+        u64 todo  = __ballot(keep);
+        while(todo)
+        {
+            int leader = __ffsll((long long)todo) - 1;
+            int el     = __shfl(e, leader);
+            u64 m      = __ballot(keep && e == el);
+            if(keep && e == el)
+            {
+                u32 pos          = base[el] + (u32)__popcll(m & lt);
+                u32 tok          = (u32)(i / a.k);
+                u32 slot         = (u32)(i - (int)tok * a.k);
+                a.sorted_ids[pos] = (slot << 24) | tok;
+                a.sorted_w[pos]   = w;
+            }
+            if(lane == leader)
+                base[el] += (u32)__popcll(m);
+            todo &= ~m;
+        }
+    }
+}
+
+// per-expert padded offsets from per-expert totals; one workgroup, any thread count that is a
+// multiple of 64.  tot[e] in, off[e] (exclusive prefix of padded sizes) and lid[e] out; returns
+// the padded total to every thread.  scratch: >= blockDim/64 + 1 words of LDS.
+__device__ __forceinline__ u32 expert_offsets(const SortArgs& a, const u32* tot, u32* off, u32* lid,
+                                              u32* scratch)
+{
+    const int nw   = blockDim.x / WAVE;
+    const int lane = lane_id(), wave = threadIdx.x / WAVE;
+    u32 run_pad = 0, run_id = 0;
+    for(int e0 = 0; e0 < a.E; e0 += blockDim.x)
+    {
+        int e     = e0 + threadIdx.x;
+        bool on   = e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
+        u32 pad   = (on && e < a.E) ? (tot[e] + a.Bm - 1) / a.Bm * a.Bm : 0u;
+        u32 one   = on ? 1u : 0u;
+        // inclusive scan inside the wave (two values packed: padded size, mask count)
+        u32 sp = pad, si = one;
+        for(int d = 1; d < WAVE; d <<= 1)
+        {
+            u32 tp = __shfl_up(sp, d), ti = __shfl_up(si, d);
+            if(lane >= d)
+            {
+                sp += tp;
+                si += ti;
+            }
+        }
+        __syncthreads();
+        if(lane == WAVE - 1)
+        {
+            scratch[wave]      = sp;
+            scratch[nw + wave] = si;
+        }
+        __syncthreads();
+        u32 bp = 0, bi = 0, allp = 0, alli = 0;
+        for(int w = 0; w < nw; w++)
+        {
+            u32 p = scratch[w], q = scratch[nw + w];
+            if(w < wave)
+            {
+                bp += p;
+                bi += q;
+            }
+            allp += p;
+            alli += q;
+        }
+        if(e < a.E)
+        {
+            off[e] = run_pad + bp + sp - pad;
+            lid[e] = a.expert_mask ? run_id + bi + si - one : (u32)e;
+        }
+        run_pad += allp;
+        run_id += alli;
+    }
+    __syncthreads();
+    return run_pad;
+}
+
+// padding entries of every expert's run, the tail past the padded total, the block -> expert
+// table and num_valid.  Touches no position that holds a real pair, so it may run concurrently
+// with the scatter.
+__device__ __forceinline__ void fill_outputs(const SortArgs& a, const u32* tot, const u32* off,
+                                             const u32* lid, u32 padded_total, int T, int tid, int nthreads)
+{
+    const u32 pad_id = ((u32)a.k << 24) | ((u32)T & 0xFFFFFFu);
+    const u32 n      = (u32)a.n_blk * (u32)a.Bm;
+    const int nwaves = nthreads / WAVE, wave = tid / WAVE, lane = tid % WAVE;
+    for(int e = wave; e < a.E; e += nwaves)
+    {
+        if(tot[e] == 0 || (a.expert_mask && a.expert_mask[e] == 0))
+            continue;
+        u32 beg = off[e] + tot[e];
+        u32 end = off[e] + (tot[e] + a.Bm - 1) / a.Bm * a.Bm;
+        for(u32 p = beg + lane; p < end; p += WAVE)
+        {
+            a.sorted_ids[p] = pad_id;
+            a.sorted_w[p]   = 0.f;
+        }
+        for(u32 b = off[e] / a.Bm + lane; b < end / a.Bm; b += WAVE)
+            a.sorted_e[b] = lid[e];
+    }
+    for(u32 p = padded_total + tid; p < n; p += nthreads)
+    {
+        a.sorted_ids[p] = pad_id;
+        a.sorted_w[p]   = 0.f;
+    }
+    for(u32 b = padded_total / a.Bm + tid; b < (u32)a.n_blk; b += nthreads)
+        a.sorted_e[b] = EXPERT_FILL;
+    if(tid == 0)
+    {
+        a.num_valid[0] = padded_total;
+        a.num_valid[1] = (u32)T;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// single workgroup: everything in one launch (decode-sized inputs)
+// LDS: whist[SMALL_WAVES][E] | tot[E] | off[E] | lid[E] | scratch[2*SMALL_WAVES]
+extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a)
+{
+    extern __shared__ u32 lds[];
+    u32* whist   = lds;
+    u32* tot     = whist + SMALL_WAVES * a.E;
+    u32* off     = tot + a.E;
+    u32* lid     = off + a.E;
+    u32* scratch = lid + a.E;
+    const int T     = sort_tokens(a);
+    const int pairs = T * a.k;
+    const int wave  = threadIdx.x / WAVE;
+    const int cv    = wave_chunk(pairs, SMALL_WAVES);
+    const int beg   = min(pairs, wave * cv), end = min(pairs, beg + cv);
+
+    for(int i = threadIdx.x; i < SMALL_WAVES * a.E; i += SMALL_THREADS)
+        whist[i] = 0;
+    __syncthreads();
+    wave_hist(a, whist + wave * a.E, beg, end);
+    __syncthreads();
+    // exclusive prefix over waves, per expert
+    for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
+    {
+        u32 run = 0;
+        for(int w = 0; w < SMALL_WAVES; w++)
+        {
+            u32 c             = whist[w * a.E + e];
+            whist[w * a.E + e] = run;
+            run += c;
+        }
+        tot[e] = run;
+    }
+    __syncthreads();
+    u32 padded_total = expert_offsets(a, tot, off, lid, scratch);
+    fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+    for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
+        for(int w = 0; w < SMALL_WAVES; w++)
+            whist[w * a.E + e] += off[e];
+    __syncthreads();
+    wave_scatter(a, whist + wave * a.E, beg, end);
+}
+
+// ---------------------------------------------------------------------------------------------
+// large inputs, launch 1 of 3: per-workgroup histogram -> ws[g][E]
+extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_hist_kernel(SortArgs a)
+{
+    extern __shared__ u32 lds[];
+    const int T     = sort_tokens(a);
+    const int pairs = T * a.k;
+    const int cv    = wave_chunk(pairs, a.G * SORT_WAVES);
+    const int wid   = blockIdx.x * SORT_WAVES + threadIdx.x / WAVE;
+    const int beg   = min(pairs, wid * cv), end = min(pairs, beg + cv);
+    for(int i = threadIdx.x; i < a.E; i += SORT_THREADS)
+        lds[i] = 0;
+    __syncthreads();
+    wave_hist(a, lds, beg, end);
+    __syncthreads();
+    for(int i = threadIdx.x; i < a.E; i += SORT_THREADS)
+        a.ws[(size_t)blockIdx.x * a.E + i] = lds[i];
+}
+
+// launch 2 of 3 (one workgroup): ws[g][e] -> exclusive prefix over g; offsets; padding; tables
+// LDS: tot[E] | off[E] | lid[E] | scratch
+extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel(SortArgs a)
+{
+    extern __shared__ u32 lds[];
+    u32* tot     = lds;
+    u32* off     = tot + a.E;
+    u32* lid     = off + a.E;
+    u32* scratch = lid + a.E;
+    const int T  = sort_tokens(a);
+    for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
+    {
+        u32 run = 0;
+        for(int g = 0; g < a.G; g++)
+        {
+            u32 c                    = a.ws[(size_t)g * a.E + e];
+            a.ws[(size_t)g * a.E + e] = run;
+            run += c;
+        }
+        tot[e] = run;
+    }
+    __syncthreads();
+    u32 padded_total = expert_offsets(a, tot, off, lid, scratch);
+    u32* g_off       = a.ws + (size_t)a.G * a.E;
+    for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
+        g_off[e] = off[e];
+    fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+}
+
+// launch 3 of 3: scatter.  LDS: whist[SORT_WAVES][E]
+extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_scatter_kernel(SortArgs a)
+{
+    extern __shared__ u32 lds[];
+    const int T     = sort_tokens(a);
+    const int pairs = T * a.k;
+    const int cv    = wave_chunk(pairs, a.G * SORT_WAVES);
+    const int wave  = threadIdx.x / WAVE;
+    const int wid   = blockIdx.x * SORT_WAVES + wave;
+    const int beg   = min(pairs, wid * cv), end = min(pairs, beg + cv);
+    for(int i = threadIdx.x; i < SORT_WAVES * a.E; i += SORT_THREADS)
+        lds[i] = 0;
+    __syncthreads();
+    wave_hist(a, lds + wave * a.E, beg, end);
+    __syncthreads();
+    const u32* g_off = a.ws + (size_t)a.G * a.E;
+    for(int e = threadIdx.x; e < a.E; e += SORT_THREADS)
+    {
+        u32 run = g_off[e] + a.ws[(size_t)blockIdx.x * a.E + e];
+        for(int w = 0; w < SORT_WAVES; w++)
+        {
+            u32 c            = lds[w * a.E + e];
+            lds[w * a.E + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    wave_scatter(a, lds + wave * a.E, beg, end);
+}
+
+// zero fill of the layer output buffer the reference's sorter hands back
+extern "C" __global__ void moe_zero_kernel(uint4* p, size_t n16, unsigned char* tail, int ntail)
+{
+    size_t i      = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for(; i < n16; i += stride)
+        p[i] = make_uint4(0, 0, 0, 0);
+    if(blockIdx.x == 0 && (int)threadIdx.x < ntail)
+        tail[threadIdx.x] = 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+#define SMALL_PAIRS_MAX 4096
+#define MAX_EXPERTS 2048
+
+static int sort_groups(int64_t pairs)
+{
+    // workgroups of the large path: 256 pairs per wave-chunk minimum, at most 128 workgroups
+    int64_t g = (pairs + SORT_THREADS * 4 - 1) / (SORT_THREADS * 4);
+    return (int)(g < 1 ? 1 : (g > 128 ? 128 : g));
+}
+
+extern "C" int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size)
+{
+    return (tokens * topk + (int64_t)experts * (block_size - 1) + block_size - 1) / block_size;
+}
+
+extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, int experts)
+{
+    int64_t pairs = tokens * topk;
+    if(pairs <= SMALL_PAIRS_MAX)
+        return 256;
+    return ((int64_t)sort_groups(pairs) + 1) * experts * 4 + 256;
+}
+
+extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
+                                 int experts, int block_size, const int32_t* expert_mask,
+                                 const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
+                                 uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, void* moe_out,
+                                 int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
+                                 hipStream_t stream)
+{
+    PYHIP_REQUIRE(topk_ids && topk_weights && sorted_ids && sorted_weights && sorted_expert_ids && num_valid_ids,
+                  "moe_sorting: null pointer");
+    PYHIP_REQUIRE(tokens >= 0 && tokens < (1 << 24), "moe_sorting: tokens=%d outside [0, 2^24)", tokens);
+    PYHIP_REQUIRE(topk >= 1 && topk <= 255, "moe_sorting: topk=%d outside [1, 255]", topk);
+    PYHIP_REQUIRE(experts >= 1 && experts <= MAX_EXPERTS, "moe_sorting: experts=%d outside [1, %d]", experts,
+                  MAX_EXPERTS);
+    PYHIP_REQUIRE(block_size >= 1, "moe_sorting: block_size=%d", block_size);
+    int64_t pairs = (int64_t)tokens * topk;
+    PYHIP_REQUIRE(pairs + (int64_t)experts * block_size < (1ll << 31), "moe_sorting: too many pairs");
+    PYHIP_REQUIRE(workspace_bytes >= pyhip_moe_sorting_workspace_bytes(tokens, topk, experts) &&
+                      (workspace || workspace_bytes == 0),
+                  "moe_sorting: workspace too small");
+    SortArgs a;
+    a.topk_ids      = topk_ids;
+    a.topk_w        = topk_weights;
+    a.expert_mask   = expert_mask;
+    a.num_local_tok = num_local_tokens;
+    a.sorted_ids    = sorted_ids;
+    a.sorted_w      = sorted_weights;
+    a.sorted_e      = sorted_expert_ids;
+    a.num_valid     = num_valid_ids;
+    a.ws            = (u32*)workspace;
+    a.T_all         = tokens;
+    a.k             = topk;
+    a.E             = experts;
+    a.Bm            = block_size;
+    a.n_blk         = (int)pyhip_moe_sorting_max_blocks(tokens, topk, experts, block_size);
+    a.G             = 1;
+    if(moe_out && moe_out_bytes > 0)
+    {
+        size_t n16 = (size_t)moe_out_bytes / 16;
+        int ntail  = (int)(moe_out_bytes - (int64_t)n16 * 16);
+        int grid   = (int)((n16 + 255) / 256);
+        grid       = grid < 1 ? 1 : (grid > 2048 ? 2048 : grid);
+        hipLaunchKernelGGL(moe_zero_kernel, dim3(grid), dim3(256), 0, stream, (uint4*)moe_out, n16,
+                           (unsigned char*)moe_out + n16 * 16, ntail);
+        PYHIP_CHECK_LAUNCH("moe_zero_kernel");
+    }
+    if(pairs <= SMALL_PAIRS_MAX)
+    {
+        size_t lds = ((size_t)(SMALL_WAVES + 3) * experts + 2 * SMALL_WAVES + 2) * 4;
+        if(lds > 64 * 1024)
+        {
+            hipError_t e = hipFuncSetAttribute((const void*)moe_sort_small_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            PYHIP_REQUIRE(e == hipSuccess, "moe_sorting: cannot reserve %zu B of LDS", lds);
+        }
+        hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(SMALL_THREADS), lds, stream, a);
+        PYHIP_CHECK_LAUNCH("moe_sort_small_kernel");
+        return PYHIP_OK;
+    }
+    a.G = sort_groups(pairs);
+    hipLaunchKernelGGL(moe_sort_hist_kernel, dim3(a.G), dim3(SORT_THREADS), (size_t)experts * 4, stream, a);
+    PYHIP_CHECK_LAUNCH("moe_sort_hist_kernel");
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(SMALL_THREADS),
+                       ((size_t)3 * experts + 2 * SMALL_WAVES + 2) * 4, stream, a);
+    PYHIP_CHECK_LAUNCH("moe_sort_scan_kernel");
+    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(a.G), dim3(SORT_THREADS), (size_t)SORT_WAVES * experts * 4,
+                       stream, a);
+    PYHIP_CHECK_LAUNCH("moe_sort_scatter_kernel");
+    return PYHIP_OK;
+}

@@ -1,0 +1,139 @@
+"""``fused_moe``: MXFP4 fused Mixture-of-Experts layer on MI355X.
+
+Same call surface as the reference's ``fused_moe`` (src/contrib/fused_moe.py:128-155): routing weights
+and top-k ids in, per-token bf16 hidden states out.  Weights are MXFP4 (``quant_type=QuantType.per_1x32``):
+``w1`` [E, 2*I, H/2] (gate rows then up rows) and ``w2`` [E, H, I/2] as uint8 / float4_e2m1fn_x2 in the
+pre-shuffled layout, ``w1_scale`` / ``w2_scale`` e8m0 in the shuffled layout (see ``pyhip_amd.mxfp4``).
+
+Pipeline (all launches on the current torch stream, no host synchronisation):
+  sort -> quantise activations to MXFP4 -> gate_up GEMM + SiLU*up -> quantise -> down GEMM * routing
+  weight -> top-k reduction.
+"""
+import torch
+
+from . import _lib
+from .enums import ActivationType, QuantType
+from .moe_sorting import moe_sorting, max_blocks
+
+__all__ = ["fused_moe"]
+
+
+def _as_u8(t):
+    if t is None:
+        return None
+    return t if t.dtype == torch.uint8 else t.view(torch.uint8)
+
+
+def pick_block_m(tokens, topk, experts):
+    """M-tile (= sort block size): the smallest tile that holds the expected rows per expert."""
+    est = tokens * topk / max(experts, 1)
+    for bm in (16, 32, 64):
+        if est <= bm:
+            return bm
+    return 128
+
+
+def act_quant_mxfp4(x, rows_limit=None):
+    """bf16 [rows, K] -> (uint8 [rows, K/2], uint8 [rows, ceil(K/512)*16]) in the GEMM's A-operand layout."""
+    lib = _lib.load()
+    assert x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
+    rows, K = x.shape
+    sk = lib.pyhip_moe_act_scale_stride(K)
+    q = torch.empty(rows, K // 2, dtype=torch.uint8, device=x.device)
+    s = torch.empty(rows, sk, dtype=torch.uint8, device=x.device)
+    rc = lib.pyhip_moe_act_quant_mxfp4(_lib.dptr(x), x.stride(0), rows, K, _lib.dptr(q), _lib.dptr(s),
+                                       _lib.dptr(rows_limit), _lib.current_stream())
+    _lib.check(rc, "act_quant_mxfp4")
+    return q, s
+
+
+def fused_moe(
+    hidden_states,
+    w1,  # [E, inter_dim*2, dim/2]  gate rows then up rows
+    w2,  # [E, dim, inter_dim/2]
+    topk_weight,
+    topk_ids,
+    expert_mask=None,
+    activation=ActivationType.Silu,
+    quant_type=QuantType.per_1x32,
+    doweight_stage1=False,
+    w1_scale=None,
+    w2_scale=None,
+    a1_scale=None,
+    a2_scale=None,
+    block_size_M=None,
+    num_local_tokens=None,
+    moe_sorting_dispatch_policy=0,
+    dtype=None,
+    hidden_pad=0,
+    intermediate_pad=0,
+    bias1=None,
+    bias2=None,
+    splitk=0,
+    method="auto",
+    return_parts=False,
+):
+    lib = _lib.load()
+    assert activation == ActivationType.Silu, "only SiLU-gated experts are implemented"
+    assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
+    assert not doweight_stage1
+    assert a1_scale is None and a2_scale is None, "activations are quantised dynamically"
+    assert hidden_pad == 0 and intermediate_pad == 0
+    assert splitk == 0
+    assert w1_scale is not None and w2_scale is not None
+    assert hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2
+    out_dtype = hidden_states.dtype if dtype is None else dtype
+    assert out_dtype in (torch.bfloat16, torch.float32)
+
+    w1u, w2u, w1s, w2s = _as_u8(w1), _as_u8(w2), _as_u8(w1_scale), _as_u8(w2_scale)
+    T, H = hidden_states.shape
+    k = topk_ids.shape[1]
+    E, N1, Hb = w1u.shape
+    I = N1 // 2
+    assert Hb * 2 == H and tuple(w2u.shape) == (E, H, I // 2), (w1u.shape, w2u.shape, H)
+    assert w1u.is_contiguous() and w2u.is_contiguous() and w1s.is_contiguous() and w2s.is_contiguous()
+    global_E = E if expert_mask is None else expert_mask.numel()
+    dev = hidden_states.device
+    if T == 0:
+        return torch.zeros(0, H, dtype=out_dtype, device=dev)
+
+    topk_ids = topk_ids.to(torch.int32).contiguous()
+    topk_weight = topk_weight.to(torch.float32).contiguous()
+    bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
+    sorted_ids, sorted_w, sorted_e, num_valid, _ = moe_sorting(
+        topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
+        moe_sorting_dispatch_policy, alloc_moe_out=False)
+    n_blk = sorted_e.numel()
+    stream = _lib.current_stream()
+
+    if bias1 is not None:
+        bias1 = bias1.to(torch.bfloat16).contiguous()
+        assert tuple(bias1.shape) == (E, 2 * I)
+    if bias2 is not None:
+        bias2 = bias2.to(torch.bfloat16).contiguous()
+        assert tuple(bias2.shape) == (E, H)
+
+    a1_q, a1_s = act_quant_mxfp4(hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous())
+    a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
+    rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
+                                   _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
+                                   _lib.dptr(num_valid), _lib.dptr(a2), T, k, E, H, I, bm, n_blk, stream)
+    _lib.check(rc, "moe_gemm1_mxfp4")
+    a2_q, a2_s = act_quant_mxfp4(a2, rows_limit=num_valid)
+    out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
+    if expert_mask is not None or num_local_tokens is not None:
+        out3.zero_()          # slots routed to experts this rank does not hold contribute nothing
+    rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                   _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                   _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(out3),
+                                   T, k, E, H, I, bm, n_blk, stream)
+    _lib.check(rc, "moe_gemm2_mxfp4")
+    out = torch.empty(T, H, dtype=out_dtype, device=dev)
+    rc = lib.pyhip_moe_topk_reduce(_lib.dptr(out3), _lib.dptr(out), T, k, H,
+                                   1 if out_dtype == torch.float32 else 0, None, stream)
+    _lib.check(rc, "moe_topk_reduce")
+    if return_parts:
+        return out, dict(sorted_ids=sorted_ids, sorted_weights=sorted_w, sorted_expert_ids=sorted_e,
+                         num_valid_ids=num_valid, a1_q=a1_q, a1_s=a1_s, a2=a2, a2_q=a2_q, a2_s=a2_s,
+                         out3=out3, block_m=bm)
+    return out

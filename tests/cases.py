@@ -1,0 +1,65 @@
+"""Seeded synthetic MoE layers for the tests.  Inputs are drawn with a CPU generator so that the
+build container and the GPU box see identical data; weights are quantised with the ORACLE's numpy
+quantiser (the product's torch quantiser is checked against it separately)."""
+import numpy as np
+import torch
+
+from oracle import layout, mxfp4, routing
+
+CONFIGS = {
+    # name: E, topk, H, I, router
+    "tiny": dict(E=8, k=2, H=1024, I=512, router="softmax"),
+    "mixtral_s": dict(E=8, k=2, H=1024, I=1024, router="softmax"),          # Mixtral-shaped, scaled down
+    "qwen3_s": dict(E=32, k=8, H=1024, I=512, router="zipf"),
+    "dsv3_s": dict(E=64, k=8, H=1024, I=512, router="grouped"),
+}
+
+
+class Layer:
+    pass
+
+
+def make_layer(name, T, seed=0, bias=False, E=None, k=None, H=None, I=None, router=None):
+    cfg = dict(CONFIGS[name]) if name in CONFIGS else {}
+    for key, v in dict(E=E, k=k, H=H, I=I, router=router).items():
+        if v is not None:
+            cfg[key] = v
+    E, k, H, I = cfg["E"], cfg["k"], cfg["H"], cfg["I"]
+    g = torch.Generator().manual_seed(seed)
+    L = Layer()
+    L.E, L.k, L.H, L.I, L.T = E, k, H, I, T
+    L.hidden = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(E, 2 * I, H, generator=g) * 0.02).numpy()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.02).numpy()
+    L.w1q, L.w1s = mxfp4.quantize_mxfp4(w1)
+    L.w2q, L.w2s = mxfp4.quantize_mxfp4(w2)
+    logits = torch.randn(T, E, generator=g).numpy().astype(np.float64)
+    if cfg["router"] == "softmax":
+        L.topk_w, L.topk_ids = routing.softmax_topk(logits, k)
+    elif cfg["router"] == "zipf":
+        zb = np.log(1.0 / np.arange(1, E + 1) ** 1.1)
+        L.topk_w, L.topk_ids = routing.softmax_topk(logits + zb[None, :] - zb.mean(), k)
+    else:
+        L.topk_w, L.topk_ids = routing.grouped_sigmoid_topk(logits, k, n_group=8, topk_group=4)
+    L.bias1 = L.bias2 = None
+    if bias:
+        L.bias1 = (torch.randn(E, 2 * I, generator=g) * 0.01).to(torch.bfloat16)
+        L.bias2 = (torch.randn(E, H, generator=g) * 0.01).to(torch.bfloat16)
+    return L
+
+
+def device_weights(L, dev="cuda"):
+    """shuffled device tensors in the layout fused_moe takes"""
+    w1 = torch.from_numpy(layout.shuffle_weight(L.w1q)).to(dev)
+    w2 = torch.from_numpy(layout.shuffle_weight(L.w2q)).to(dev)
+    w1s = torch.from_numpy(layout.e8m0_shuffle(L.w1s.reshape(L.E * 2 * L.I, L.H // 32))).to(dev)
+    w2s = torch.from_numpy(layout.e8m0_shuffle(L.w2s.reshape(L.E * L.H, L.I // 32))).to(dev)
+    return w1, w1s, w2, w2s
+
+
+def untranspose_act_scales(s, K):
+    """kernel activation-scale layout [rows, SK] -> plain [rows, K/32] (numpy)"""
+    rows, SK = s.shape
+    g = s.reshape(rows, SK // 16, 4, 4)            # [q][kb][i]  ->  block 16q + 4i + kb
+    plain = g.transpose(0, 1, 3, 2).reshape(rows, SK)
+    return plain[:, : K // 32]

@@ -1,0 +1,58 @@
+"""CPU checks of the boundary: the shared library loads and exports every symbol that
+include/pyhip_moe.h declares, the ctypes table covers exactly those symbols, and the argument
+checks reject bad input without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from pyhip_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "pyhip_moe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pyhip_moe_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.pyhip_moe_abi_version() == 1
+
+
+def test_size_helpers():
+    lib = _lib.load()
+    assert lib.pyhip_moe_sorting_max_blocks(64, 2, 8, 16) == (128 + 8 * 15 + 15) // 16
+    assert lib.pyhip_moe_act_scale_stride(7168) == 224 and lib.pyhip_moe_act_scale_stride(1024) == 32
+    assert lib.pyhip_moe_act_scale_stride(2880) == 96
+    assert lib.pyhip_moe_sorting_workspace_bytes(16, 8, 256) >= 0
+
+
+def test_argument_errors_are_reported():
+    lib = _lib.load()
+    rc = lib.pyhip_moe_sorting(None, None, 4, 2, 8, 16, None, None, None, None, None, None, None, 0, None, 0, None)
+    assert rc == 1
+    with pytest.raises(_lib.PyhipError, match="null pointer"):
+        _lib.check(rc, "moe_sorting")
+    one = ctypes.c_void_p(16)
+    rc = lib.pyhip_moe_act_quant_mxfp4(one, 40, 4, 40, one, one, None, None)
+    assert rc == 1 and b"multiple of 32" in lib.pyhip_moe_last_error()
+    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, one, 4, 2, 8, 1000, 512, 16, 4, None)
+    assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
+    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, one, 4, 2, 8, 1024, 512, 48, 4, None)
+    assert rc == 1 and b"block_m" in lib.pyhip_moe_last_error()
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libpyhip_moe.so")
+    with pytest.raises(_lib.PyhipError, match="no fallback"):
+        _lib.load()

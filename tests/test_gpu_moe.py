@@ -1,0 +1,139 @@
+"""GPU parity of the MXFP4 fused-MoE hot path through the C ABI.
+
+Tolerance (floating point): against the oracle's fp32 path on identical seeded inputs,
+max|err| <= 1e-2 * rms(ref) and cosine >= 0.999 on the operator's fp32 output; its bf16 output may
+differ from the fp32 reference by half a bf16 ulp of the value on top of that (the output quantum).
+Integer/byte stages (activation quantisation, sort) are bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import metrics, moe, mxfp4 as om
+from pyhip_amd import fused_moe
+from pyhip_amd.fused_moe import act_quant_mxfp4
+import cases
+
+pytestmark = pytest.mark.gpu
+
+TOL_MAX = 1e-2
+TOL_COS = 0.999
+
+
+def _f(t):
+    return t.float().cpu().numpy()
+
+
+def test_act_quant_bit_exact():
+    g = torch.Generator().manual_seed(0)
+    rows, K = 37, 1024
+    x = torch.randn(rows, K, generator=g) * torch.exp(torch.randn(rows, 1, generator=g) * 3)
+    x[0, :32] = 0                                                     # all-zero block
+    ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 4.0, -0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0, 6.0])
+    x[1, :16] = ties                                                  # exact ties, block scale 1
+    x[1, 16:32] = 0
+    x[2, :32] = torch.linspace(-7.9, 7.9, 32)                         # saturation range (scale 1)
+    x[3, :64] = torch.randn(64, generator=g) * 1e-30                  # tiny exponents
+    x[4, :64] = torch.randn(64, generator=g) * 1e30
+    xb = x.to(torch.bfloat16)
+    print("act_quant case rows=37 K=1024", flush=True)
+    q, s = act_quant_mxfp4(xb.cuda())
+    torch.cuda.synchronize()
+    oq, os_ = om.quantize_mxfp4(xb.float().numpy())
+    got_s = cases.untranspose_act_scales(s.cpu().numpy(), K)
+    assert (got_s == os_).all(), np.argwhere(got_s != os_)[:10]
+    bad = np.argwhere(q.cpu().numpy() != oq)
+    assert bad.size == 0, (bad[:10], q.cpu().numpy()[tuple(bad[0])], oq[tuple(bad[0])])
+
+
+def _stage_checks(L, parts, bm):
+    """stage-by-stage comparison; every stage is fed the KERNEL's previous output."""
+    so = parts["sorted_ids"].cpu().numpy().view(np.uint32)
+    se = parts["sorted_expert_ids"].cpu().numpy().view(np.uint32)
+    sw = parts["sorted_weights"].cpu().numpy()
+    nv = int(parts["num_valid_ids"][0])
+    x = om.dequantize_mxfp4(*om.quantize_mxfp4(_f(L.hidden)))
+    a2 = _f(parts["a2"])
+    out3 = _f(parts["out3"])
+    a2q = om.dequantize_mxfp4(*om.quantize_mxfp4(a2[:nv]))
+    worst1 = worst2 = 0.0
+    nflip1 = nflip2 = ntot1 = ntot2 = 0
+    for b in range(nv // bm):
+        e = int(se[b])
+        ids = so[b * bm:(b + 1) * bm]
+        tok, slot = (ids & 0xFFFFFF).astype(np.int64), (ids >> 24).astype(np.int64)
+        ok = slot < L.k
+        w1 = moe.expert_weights_f32(L.w1q[e], L.w1s[e])
+        w2 = moe.expert_weights_f32(L.w2q[e], L.w2s[e])
+        b1 = None if L.bias1 is None else _f(L.bias1[e])
+        b2 = None if L.bias2 is None else _f(L.bias2[e])
+        ref1 = moe.gateup_ref(x[tok[ok]], w1, b1)
+        got1 = a2[b * bm:(b + 1) * bm][ok]
+        rms1 = np.sqrt(np.mean(ref1 ** 2)) + 1e-30
+        # both sides are bf16 roundings of nearly equal fp32 values: allow one bf16 ulp of the value
+        worst1 = max(worst1, (np.maximum(np.abs(got1 - ref1) - np.abs(ref1) * 2.0 ** -7, 0)).max() / rms1)
+        nflip1 += int((got1 != ref1).sum())
+        ntot1 += got1.size
+        assert (a2[b * bm:(b + 1) * bm][~ok] == 0).all()
+        ref2 = moe.down_ref(a2q[b * bm:(b + 1) * bm][ok], w2, sw[b * bm:(b + 1) * bm][ok], b2)
+        got2 = out3[tok[ok], slot[ok]]
+        rms2 = np.sqrt(np.mean(ref2 ** 2)) + 1e-30
+        worst2 = max(worst2, (np.maximum(np.abs(got2 - ref2) - np.abs(ref2) * 2.0 ** -7, 0)).max() / rms2)
+        nflip2 += int((got2 != ref2).sum())
+        ntot2 += got2.size
+    # one-ulp disagreements must stay rare
+    assert nflip1 <= 0.02 * ntot1 and nflip2 <= 0.02 * ntot2, (nflip1, ntot1, nflip2, ntot2)
+    return worst1, worst2
+
+
+@pytest.mark.parametrize("name,T,bm,bias", [
+    ("tiny", 64, None, False),        # BASELINE config 0
+    ("tiny", 64, 16, False),
+    ("tiny", 64, 32, True),
+    ("tiny", 5, 16, False),
+    ("tiny", 300, 64, False),
+    ("tiny", 300, 128, True),
+    ("mixtral_s", 33, 32, False),
+    ("qwen3_s", 64, 16, False),
+    ("qwen3_s", 257, 64, False),
+    ("dsv3_s", 16, 16, False),
+    ("dsv3_s", 128, None, False),
+])
+def test_fused_moe_matches_oracle(name, T, bm, bias):
+    L = cases.make_layer(name, T, seed=0, bias=bias)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    b1 = None if L.bias1 is None else L.bias1.cuda()
+    b2 = None if L.bias2 is None else L.bias2.cuda()
+    print(f"fused_moe case {name} T={T} bm={bm} bias={bias}", flush=True)
+    out32, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
+                             bias1=b1, bias2=b2, dtype=torch.float32, return_parts=True)
+    out16 = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
+                      bias1=b1, bias2=b2)
+    torch.cuda.synchronize()
+    assert out16.dtype == torch.bfloat16 and out16.shape == (T, L.H)
+
+    # activation quantisation: bit-exact
+    oq, os_ = om.quantize_mxfp4(_f(L.hidden))
+    assert (parts["a1_q"].cpu().numpy() == oq).all()
+    assert (cases.untranspose_act_scales(parts["a1_s"].cpu().numpy(), L.H) == os_).all()
+
+    # stage-wise, each stage fed the kernel's own previous output
+    w1e, w2e = _stage_checks(L, parts, parts["block_m"])
+    assert w1e <= TOL_MAX, f"stage 1 (max|err| - ulp)/rms = {w1e}"
+    assert w2e <= TOL_MAX, f"stage 2 (max|err| - ulp)/rms = {w2e}"
+
+    # end to end
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4",
+                      bias1=None if L.bias1 is None else _f(L.bias1), bias2=None if L.bias2 is None else _f(L.bias2))
+    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+    got32 = _f(out32)
+    err = metrics.max_err_over_rms(got32, ref)
+    cos = metrics.cosine(got32, ref)
+    print(f"  max|err|/rms={err:.3e} cosine={cos:.8f} calc_diff={metrics.calc_diff(got32, ref):.3e}", flush=True)
+    assert cos >= TOL_COS
+    assert err <= TOL_MAX
+    half_ulp = np.abs(ref) * 2.0 ** -8
+    assert (np.abs(_f(out16) - ref) <= TOL_MAX * rms + half_ulp).all()
+    # the bf16 output is the rounding of the fp32 output
+    assert (_f(out16) == om.bf16_round(got32)).all()
