@@ -72,7 +72,11 @@ def fused_moe(
     splitk=0,
     method="auto",
     return_parts=False,
+    stage_events=None,
 ):
+    """See the module docstring.  Extras beyond the reference signature: ``dtype=torch.float32`` returns
+    the fp32 top-k sum without the final bf16 rounding; ``return_parts=True`` also returns the
+    intermediate buffers; ``stage_events`` (a list) receives ``(name, start_event, end_event)`` per stage."""
     lib = _lib.load()
     assert activation == ActivationType.Silu, "only SiLU-gated experts are implemented"
     assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
@@ -97,12 +101,23 @@ def fused_moe(
     if T == 0:
         return torch.zeros(0, H, dtype=out_dtype, device=dev)
 
+    def _mark(name, start=None):
+        if stage_events is None:
+            return None
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        if start is not None:
+            stage_events.append((name, start, ev))
+        return ev
+
     topk_ids = topk_ids.to(torch.int32).contiguous()
     topk_weight = topk_weight.to(torch.float32).contiguous()
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
+    ev = _mark("start")
     sorted_ids, sorted_w, sorted_e, num_valid, _ = moe_sorting(
         topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
         moe_sorting_dispatch_policy, alloc_moe_out=False)
+    ev = _mark("sort", ev)
     n_blk = sorted_e.numel()
     stream = _lib.current_stream()
 
@@ -115,23 +130,28 @@ def fused_moe(
 
     a1_q, a1_s = act_quant_mxfp4(hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous())
     a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
+    ev = _mark("quant1", ev)
     rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                    _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
                                    _lib.dptr(num_valid), _lib.dptr(a2), T, k, E, H, I, bm, n_blk, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
+    ev = _mark("gemm1", ev)
     a2_q, a2_s = act_quant_mxfp4(a2, rows_limit=num_valid)
     out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
     if expert_mask is not None or num_local_tokens is not None:
         out3.zero_()          # slots routed to experts this rank does not hold contribute nothing
+    ev = _mark("quant2", ev)
     rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
                                    _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
                                    _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(out3),
                                    T, k, E, H, I, bm, n_blk, stream)
     _lib.check(rc, "moe_gemm2_mxfp4")
+    ev = _mark("gemm2", ev)
     out = torch.empty(T, H, dtype=out_dtype, device=dev)
     rc = lib.pyhip_moe_topk_reduce(_lib.dptr(out3), _lib.dptr(out), T, k, H,
                                    1 if out_dtype == torch.float32 else 0, None, stream)
     _lib.check(rc, "moe_topk_reduce")
+    _mark("reduce", ev)
     if return_parts:
         return out, dict(sorted_ids=sorted_ids, sorted_weights=sorted_w, sorted_expert_ids=sorted_e,
                          num_valid_ids=num_valid, a1_q=a1_q, a1_s=a1_s, a2=a2, a2_q=a2_q, a2_s=a2_s,
