@@ -40,14 +40,20 @@ const char* pyhip_moe_last_error(void);
  * [experts], may be NULL) drops the pairs of masked experts and makes expert ids local;
  * num_local_tokens (device int32 scalar, may be NULL) limits the tokens that are read.
  * moe_out (may be NULL) is zero-filled over moe_out_bytes, as the reference's sorter does for the
- * layer output.  workspace: pyhip_moe_sorting_workspace_bytes() bytes of device memory. */
+ * layer output.  workspace: pyhip_moe_sorting_workspace_bytes() bytes of device memory.
+ * schedule (may be NULL; pyhip_moe_schedule_words(experts) u32 words) receives the tile schedule the
+ * grouped GEMMs below walk as a persistent grid: experts are dealt to the 8 XCDs (e % 8) and every
+ * XCD gets the prefix sums of its experts' row-block counts plus each expert's first row block.  It has
+ * no counterpart in the reference, which launches one workgroup per (tile, worst-case block)
+ * (src/contrib/moe_gemm_mxfp4.py:1000-1011). */
 int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size);
 int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, int experts);
+int64_t pyhip_moe_schedule_words(int experts);
 int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk, int experts,
                       int block_size, const int32_t* expert_mask, const int32_t* num_local_tokens,
                       uint32_t* sorted_ids, float* sorted_weights, uint32_t* sorted_expert_ids,
-                      uint32_t* num_valid_ids, void* moe_out, int64_t moe_out_bytes, void* workspace,
-                      int64_t workspace_bytes, pyhip_stream_t stream);
+                      uint32_t* num_valid_ids, uint32_t* schedule, void* moe_out, int64_t moe_out_bytes,
+                      void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Dynamic MXFP4 quantisation of bf16 activations (1x32 blocks, e8m0 scale
@@ -72,11 +78,14 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
  *   w1_scale     e8m0, shuffled as tests/contrib/moe/test_fused_moe.py:222-236 over [experts*2*inter, hidden/32]
  *   bias1        bf16 [experts, 2*inter] or NULL
  *   a2           bf16 [n_blk*block_m, inter], row = sorted position (padding rows are zero)
- * block_m must equal the block_size the sort ran with; hidden % 512 == 0, inter % 128 == 0. */
+ * block_m must equal the block_size the sort ran with and `experts` the expert count it ran with;
+ * hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
+ * workgroup per tile and worst-case block is launched, as the reference does). */
 int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
-                          const uint32_t* num_valid_ids, void* a2_bf16, int tokens, int topk, int experts,
-                          int hidden, int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
+                          const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, int tokens,
+                          int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
+                          pyhip_stream_t stream);
 
 /* Stage 2: down grouped GEMM, times the routing weight.  Replaces moe_gemm_mxfp4(gate_up=False),
  * src/contrib/moe_gemm_mxfp4.py:1291-1333 (launch: tests/contrib/moe/test_moe.py:751-763).
@@ -87,9 +96,9 @@ int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint
  * inter % 512 == 0, hidden % 256 == 0. */
 int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
                           const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
-                          const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* out3_bf16,
-                          int tokens, int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
-                          pyhip_stream_t stream);
+                          const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
+                          const uint32_t* schedule, void* out3_bf16, int tokens, int topk, int experts, int hidden,
+                          int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.

@@ -60,7 +60,7 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
 // compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})
 template <typename F, int... Is>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>)
+__device__ __forceinline__ __attribute__((always_inline)) void static_for_impl(F&& f, std::integer_sequence<int, Is...>)
 {
     (f(std::integral_constant<int, Is>{}), ...);
 }

@@ -13,13 +13,14 @@
 // private to a wave and go HBM -> VGPR -> MFMA directly: the pre-shuffled weight layout
 // ([N/16][Kb/64][lane][16 B], src/misc.py:116-130) is exactly the operand layout, one coalesced
 // 1 KB load per 16x128 tile, prefetched four K-steps ahead in a register ring.  Activation tiles
-// are shared by the 4 waves: they are DMA'd (buffer_load ... lds, 16 B per lane) three K-steps
-// ahead into a ring of four LDS stages, already in operand order (lane-linear 1 KB blocks), so
-// the ds_read_b128 of a tile is conflict-free and needs no swizzle.
+// are shared by the 4 waves: they are DMA'd (buffer_load ... lds, 16 B per lane) one K-group (four
+// K-steps) ahead into two LDS stages, row-major with an XOR swizzle of the 16 B chunks, so that both
+// the DMA (64 contiguous bytes per four lanes) and the ds_read_b128 of an operand are at full rate.
 //
 // The weight tile is the MFMA's first operand and the activation tile the second, so a lane ends
 // up with 4 consecutive output channels of one row (lane%16 = row, lane/16*4.. = channels).
 #include "common.h"
+#include <stdlib.h>
 
 #define GEMM_THREADS 256
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -35,23 +36,80 @@ struct GemmArgs
     const float* sorted_w;     // [n_blk * BM]
     const u32* sorted_e;       // [n_blk]
     const u32* num_valid;      // [2]
+    const u32* sched;          // tile schedule written by the sort (moe_sort.hip: write_schedule) or null
     void* out;                 // stage 1: bf16 [n_blk*BM, N/2]; stage 2: bf16 [T, topk, N]
-    int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows;
+    int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
+#ifdef PYHIP_GEMM_DEBUG
+    int dbg;
+    unsigned long long* dbg_t;   // [gridDim][8] accumulated phase times (100 MHz ticks)
+#endif
 };
 
+// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales; OPW / OPA select
+// the byte of the scale dwords.  Written in assembly with the accumulator tied to the destination: left to
+// the compiler, about a third of the accumulators get renamed on every K-step and the kernel no longer fits
+// its register budget.
 template <int OPW, int OPA>
-__device__ __forceinline__ v4f mfma_fp4(v4i w, v4i a, v4f c, int w_scale, int a_scale)
+__device__ __forceinline__ void mfma_fp4(v4f& acc, v4i w, v4i a, int w_scale, int a_scale)
 {
-    v8i W = {w.x, w.y, w.z, w.w, 0, 0, 0, 0};
-    v8i A = {a.x, a.y, a.z, a.w, 0, 0, 0, 0};
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W, A, c, 4, 4, OPW, w_scale, OPA, a_scale);
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4 blgp:4"
+                 : "+v"(acc)
+                 : "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1), "n"(OPW >> 1), "n"(OPA >> 1));
 }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, u32 bytes)
+// ---- vector-memory primitives.  Every VMEM operation of the pipeline is issued through inline assembly
+// and every wait on the VMEM counter is written by hand: the counter retires loads in issue order, the
+// issue order below is fixed, so "all but the N youngest operations have completed" is exact.  (Left to
+// the compiler, the waits around loop back-edges and around LDS-DMA operations collapse the prefetch
+// distance to one or two K-steps.)
+__device__ __forceinline__ v4i make_rsrc(const void* p, u32 bytes)
 {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+    const unsigned long long a = (unsigned long long)p;
+    // raw buffer: base[47:0], stride 0, num_records = bytes, word 3 = 32-bit data format
+    return (v4i){(int)(u32)a, (int)((a >> 32) & 0xFFFFu), (int)bytes, 0x00020000};
 }
-
+// address = rsrc.base + voff + soff + IMM (IMM < 4096); only voff + IMM is range-checked
+template <int IMM = 0>
+__device__ __forceinline__ void vm_load_b128(v4i& dst, int voff, v4i rsrc, int soff)
+{
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+}
+template <int IMM = 0>
+__device__ __forceinline__ void vm_load_b32(int& dst, int voff, v4i rsrc, int soff)
+{
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+}
+// global -> LDS without passing through registers: lane i's bytes land at lds_base + LDS_IMM + i * size.
+// (The hardware adds the instruction's immediate offset to the LDS address as well as to the global one, so
+// M0 is set to the target minus IMM.)
+template <int IMM, int LDS_IMM>
+__device__ __forceinline__ void vm_dma_b128(int voff, v4i rsrc, int soff, u32 lds_base)
+{
+    asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen offset:%4 lds"
+                 ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
+}
+template <int IMM, int LDS_IMM>
+__device__ __forceinline__ void vm_dma_b32(int voff, v4i rsrc, int soff, u32 lds_base)
+{
+    asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen offset:%4 lds"
+                 ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
+}
+__device__ __forceinline__ u32 lds_addr_of(const void* p)
+{
+    return (u32)(unsigned long long)(__attribute__((address_space(3))) const void*)p;
+}
+// all but the N youngest VMEM operations have completed; the registers named are (re)defined here, so
+// their consumers cannot be scheduled above the wait
+template <int N>
+__device__ __forceinline__ void wait_vm_tiles(v4i& a, v4i& b, v4i& c, v4i& d)
+{
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm_scales(int& a, int& b, int& c, int& d)
+{
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt_barrier()
 {
@@ -59,266 +117,586 @@ __device__ __forceinline__ void wait_vmcnt_barrier()
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// 4x4 transpose of dwords across the four 16-lane rows of a wave: in: x[j] of lane row kb;
+// out: x[c] of lane row q holds what x[q] of lane row c held.  (permlane32_swap exchanges lanes
+// 32..63 of its first operand with lanes 0..31 of its second; permlane16_swap exchanges the odd
+// 16-lane rows of its first operand with the even rows of its second.)
+__device__ __forceinline__ void transpose4x4_rows(u32 (&x)[4])
+{
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    v2u t;
+    t = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false); x[0] = t.x; x[2] = t.y;
+    t = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false); x[1] = t.x; x[3] = t.y;
+    t = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false); x[0] = t.x; x[1] = t.y;
+    t = __builtin_amdgcn_permlane16_swap(x[2], x[3], false, false); x[2] = t.x; x[3] = t.y;
+}
+
+struct TileId
+{
+    int m_blk, nt, e;   // row block, weight tile, (local) expert; all wave-uniform
+    bool valid;
+};
+
+#define SCHED_EX_MAX (2048 / 8 + 2)
+
 // STAGE 1 = gate_up, 2 = down.  MT = row groups of 16 per tile.
+//
+// The kernel is one flat software pipeline over (tile, K-group) pairs: while the MFMAs of K-group ks of a
+// tile run, the activation DMA of K-group ks+1 and the weight loads of K-steps 4(ks+1)..4(ks+1)+3 are in
+// flight; in the last K-group of a tile those prefetches already belong to the workgroup's NEXT tile, so
+// the memory pipeline never drains between tiles.  One barrier per K-group (512 K elements).  Everything
+// a tile boundary needs (schedule tables, sorted ids, routing weights) is read from LDS, so no wait on the
+// vector-memory counter ever covers the prefetches in flight.
 template <int STAGE, int MT>
 __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     constexpr int BM    = MT * 16;
-    constexpr int NA    = (MT + 3) / 4;       // activation tiles DMA'd per wave per K-step
-    constexpr int SLOTS = NA * 4;             // tile slots per LDS stage (slots >= MT are never read)
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a0[SLOTS * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a1[SLOTS * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a2[SLOTS * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a3[SLOTS * 1024];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_s0[SLOTS * 256];   // activation scales of a K-group
+    constexpr int NA    = (MT + 3) / 4;       // activation row groups DMA'd per wave
+    constexpr int SLOTS = NA * 4;             // row-group slots per LDS stage (slots >= MT are never read)
+    constexpr int NID   = (BM + 63) / 64;     // DMA ops that bring one tile's sorted ids (same for weights)
+    constexpr int MPAD  = NID * 64;           // words per meta array
+    constexpr int NM    = (2 * NID + 3) / 4;  // meta DMA ops per wave and K-group (same count in every wave)
+    // VMEM operations per wave and K-group, in issue order: NPF prefetch operations (NM meta, 5*NA activation,
+    // 4 weight-scale) spread between the MFMAs of K-step 0, and 4 weight tiles after each of the 4 K-steps.
+    // A weight tile loaded after K-step u is consumed by K-step u of the next K-group; younger than it at
+    // that point are the tiles of the later K-steps, and for u > 0 this K-group's prefetches and tiles.
+    constexpr int NPF = NM + 5 * NA + 4;
+    constexpr int PPM = (NPF + MT - 1) / MT;   // prefetch operations issued after each row group's MFMAs
+    // one LDS stage = the activation tile of a whole K-group (4 K-steps of 128) + its scales
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a0[4 * SLOTS * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a1[4 * SLOTS * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_s0[SLOTS * 256];
     __shared__ __attribute__((aligned(16))) uint8_t lds_s1[SLOTS * 256];
-    __shared__ int lds_row[SLOTS * 16];
+    __shared__ u32 lds_meta[3][2 * MPAD];     // per tile: sorted ids | routing weights; ring of 3 tiles
+    __shared__ u32 lds_dummy[64];             // where the zeros of switched-off meta DMA operations land
+    __shared__ u32 lds_pre[SCHED_EX_MAX];     // this XCD's schedule: block-count prefix,
+    __shared__ u32 lds_first[SCHED_EX_MAX];   //   first row block and
+    __shared__ u32 lds_lid[SCHED_EX_MAX];     //   local id of its experts
 
-    const int m_blk = blockIdx.x / g.n_tiles;
-    const int nt    = blockIdx.x - m_blk * g.n_tiles;
-    if((u32)(m_blk * BM) >= g.num_valid[0])
-        return;
-    const int e    = (int)g.sorted_e[m_blk];
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);   // wave-uniform: keeps descriptors and LDS bases scalar
     const int lane = tid % WAVE;
     const int r = lane & 15, kb = lane >> 4;
     const int Kb = g.K / 2;
+    const int KS = g.K / 512;
     const int I  = g.N / 2;   // stage 1 only
 
-    // source row of every tile row (stage 1: gathered token; stage 2: the sorted position itself)
-    for(int i = tid; i < SLOTS * 16; i += GEMM_THREADS)
+    // ---- tile iterator.  With a schedule the grid is persistent: workgroup w serves XCD x = w % 8 (the
+    // hardware deals consecutive workgroup ids round-robin to the XCDs) and walks that XCD's tile list
+    // with stride gridDim/8; the list is ordered expert -> weight tile -> row block, so the row blocks
+    // that share a weight tile run next to each other and every expert's data stays in one L2.
+    // Without a schedule (or when K has a single K-group): one tile per workgroup, weight tile fastest.
+    const bool persistent = g.sched != nullptr;
+    const int EX          = g.E / 8 + 2;
+    const int xcd         = blockIdx.x & 7;
+    const u32 qstride     = gridDim.x >> 3;
+    u32 q                 = blockIdx.x >> 3;
+    int ei                = 0;                        // cursor into this XCD's expert list (q only grows)
+    const u32 wgs_on_xcd  = gridDim.x >> 3;
+    u32 rounds_total      = 0;                        // rounds this XCD's tile list needs
+    if(persistent)
     {
-        int row = 0;
-        if(i < BM)
+        for(int i = tid; i < EX; i += GEMM_THREADS)
         {
-            int p = m_blk * BM + i;
-            if(STAGE == 1)
-            {
-                u32 id  = g.sorted_ids[p];
-                int tok = (int)(id & 0xFFFFFFu);
-                row     = ((int)(id >> 24) < g.topk && tok < g.T) ? tok : 0;   // padding rows read row 0; never stored
-            }
-            else
-                row = p;
+            const int e  = xcd + 8 * i;
+            lds_pre[i]   = g.sched[xcd * EX + i];
+            lds_first[i] = e < g.E ? g.sched[8 * EX + e] : 0u;
+            lds_lid[i]   = e < g.E ? g.sched[8 * EX + g.E + e] : 0u;
         }
-        lds_row[i] = row;
+        __syncthreads();
+        rounds_total = (lds_pre[EX - 1] * (u32)g.n_tiles + wgs_on_xcd - 1) / wgs_on_xcd;
     }
-    __syncthreads();
-
-    // ---- weight operand: 4 row groups of 16 rows, one buffer resource each (range = the row
-    // group's K extent, so prefetches past the end of K are dropped by the bounds check)
-    int wrow[4];
-#pragma unroll
-    for(int j = 0; j < 4; j++)
-        wrow[j] = (STAGE == 1) ? ((j >> 1) * I + nt * 128 + wave * 32 + (j & 1) * 16) : (nt * 256 + wave * 64 + j * 16);
-    __amdgpu_buffer_rsrc_t wrs[4];
-#pragma unroll
-    for(int j = 0; j < 4; j++)
-        wrs[j] = make_rsrc(g.w + ((size_t)e * g.N + wrow[j]) * Kb, (u32)(16 * Kb));
-    // weight scales: rows wrow[0], wrow[1] share a 32-row tile, so do wrow[2], wrow[3]
-    const uint8_t* wsptr[2];
-#pragma unroll
-    for(int h = 0; h < 2; h++)
-    {
-        size_t R = (size_t)e * g.N + wrow[2 * h];
-        wsptr[h] = g.w_s + (R / 32) * (size_t)(g.SC / 8) * 256 + lane * 4;
-    }
-    // ---- activation operand
-    const __amdgpu_buffer_rsrc_t ars  = make_rsrc(g.a_q, (u32)((size_t)g.a_rows * Kb));
-    const __amdgpu_buffer_rsrc_t asrs = make_rsrc(g.a_s, (u32)((size_t)g.a_rows * g.SK));
-    int a_off[NA];        // byte offset of this lane's 16 B inside a_q for K-step 0, per DMA slot
-    int as_off[NA];       // byte offset of this lane's scale dword inside a_s for K-group 0, per DMA slot
-#pragma unroll
-    for(int i = 0; i < NA; i++)
-    {
-        const int row = lds_row[(wave + 4 * i) * 16 + r];
-        a_off[i]      = row * Kb + kb * 16;
-        as_off[i]     = row * g.SK + kb * 4;
-    }
-
-    uint8_t* const stage[4]  = {lds_a0, lds_a1, lds_a2, lds_a3};
-    uint8_t* const sstage[2] = {lds_s0, lds_s1};
-    auto dma_a = [&](auto S, int kt) {
-        constexpr int s = decltype(S)::value;
-#pragma unroll
-        for(int i = 0; i < NA; i++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ars, LDS_PTR(stage[s] + (wave + 4 * i) * 1024), 16,
-                                                     a_off[i] + kt * 64, 0, 0, 0);
+    auto uni = [](u32 v) __attribute__((always_inline)) { return (u32)__builtin_amdgcn_readfirstlane((int)v); };
+    // ---- per-tile rendezvous of the workgroups of one XCD.  Tiles that share a weight tile (the row blocks of
+    // one expert) or an activation tile sit next to each other in the XCD's list, so they are in flight in the
+    // same round; meeting once per round keeps the workgroups within a K-group or two of each other, which is
+    // what lets the second reader of a line find it in the XCD's L2 (4 MB hold only a few microseconds of
+    // traffic).  The counter lives in the schedule buffer and is zeroed by the sort.  The wait is bounded: a
+    // missing workgroup costs time, never a hang.
+    u32* const rendezvous = persistent ? const_cast<u32*>(g.sched) + 8 * EX + 2 * g.E + (STAGE - 1) * 8 + xcd : nullptr;
+    u32 rounds_done       = 0;
+    auto meet = [&]() __attribute__((always_inline)) {
+        if(!persistent)
+            return;
+        rounds_done++;
+        if(tid == 0)
+        {
+            __hip_atomic_fetch_add(rendezvous, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const u32 target = rounds_done * wgs_on_xcd;
+            for(int spin = 0; spin < 4000; spin++)
+            {
+                if(__hip_atomic_load(rendezvous, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target)
+                    break;
+                __builtin_amdgcn_s_sleep(8);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
-    // one dword per lane: the scales of this lane's (row, K-block) for the 4 K-steps of K-group ks
-    auto dma_s = [&](auto S, int ks) {
-        constexpr int s = decltype(S)::value;
+    auto decode = [&](TileId& t) __attribute__((always_inline)) {
+        t.valid = false;
+        if(persistent)
+        {
+            if(q >= uni(lds_pre[EX - 1]) * (u32)g.n_tiles)
+                return;
+            while(q >= uni(lds_pre[ei + 1]) * (u32)g.n_tiles)
+                ei++;
+            const u32 p0    = uni(lds_pre[ei]);
+            const u32 nb    = uni(lds_pre[ei + 1]) - p0;
+            const u32 local = q - p0 * (u32)g.n_tiles;
+            t.nt            = (int)(local / nb);
+            t.m_blk         = (int)(uni(lds_first[ei]) + (local - (u32)t.nt * nb));
+            t.e             = (int)uni(lds_lid[ei]);
+            q += qstride;
+        }
+        else
+        {
+            if(q == 0xFFFFFFFFu)
+                return;
+            t.m_blk = blockIdx.x / g.n_tiles;
+            t.nt    = blockIdx.x - t.m_blk * g.n_tiles;
+            q       = 0xFFFFFFFFu;
+            if((u32)(t.m_blk * BM) >= uni(g.num_valid[0]))
+                return;
+            t.e = (int)uni(g.sorted_e[t.m_blk]);
+        }
+        t.valid = true;
+    };
+    // sorted ids and routing weights of a tile's rows -> LDS meta buffer `buf` (DMA, 64 rows per op, NM ops per
+    // wave; `on` = false issues the same operations with zero-range descriptors)
+    auto dma_meta = [&](const TileId& t, int buf, bool on) __attribute__((always_inline)) {
+        const v4i rid = make_rsrc(g.sorted_ids + (size_t)t.m_blk * BM, BM * 4);
+        const v4i rwt = make_rsrc(g.sorted_w + (size_t)t.m_blk * BM, BM * 4);
+#pragma unroll
+        for(int i = 0; i < NM; i++)
+        {
+            const int o     = wave + 4 * i;               // op index: [0, NID) ids, [NID, 2*NID) weights, beyond: nothing
+            const bool wts  = o >= NID;
+            const int oo    = wts ? o - NID : o;
+            const bool real = on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
+            // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
+            const v4i rs    = real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0);
+            const u32 dst   = real ? lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy);
+            vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
+        }
+    };
+
+    // ---- load side of the pipeline: descriptors and per-lane offsets of the tile being prefetched
+    // (every prefetch is issued unconditionally; when there is no tile left to prefetch the descriptors get
+    // a zero range, so the hardware drops the accesses and the instruction stream stays the same)
+    v4i wrs[2];    // weight rows of this wave: stage 1 [0] gate, [1] up (2 row groups each); stage 2 [0] all 4 groups
+    v4i wsrs[2];   // their scale tiles, same split (rows j = 0,1 share a 32-row scale tile, so do j = 2,3)
+    v4i ars, asrs; // activations and their scales
+    int a_off[NA], as_off[NA];        // this lane's byte offsets inside a_q / a_s at K = 0, per DMA slot
+    // DMA lane mapping: four consecutive lanes fetch the 64 contiguous bytes of one row and K-step (a gather
+    // with one row per lane costs four times the address-pipeline cycles).  LDS therefore holds a (row group,
+    // K-step) block row-major, 16 rows x 64 B; the 16 B chunk c of row r sits in slot c ^ (r / 4), which makes
+    // the operand reads (lane = K-block * 16 + row) conflict-free.
+    const int dma_row   = lane >> 2;
+    const int dma_chunk = (lane & 3) ^ (lane >> 4);
+    const int rd_a      = r * 64 + ((kb ^ (r >> 2)) * 16);   // operand read offset inside a 1 KB block
+    const int rd_s      = (r * 4 + kb) * 4;                  // scale dword read offset inside a 256 B block
+    auto setup_null = [&]() __attribute__((always_inline)) {
+        wrs[0] = wrs[1] = make_rsrc(g.w, 0);
+        wsrs[0] = wsrs[1] = make_rsrc(g.w_s, 0);
+        ars  = make_rsrc(g.a_q, 0);
+        asrs = make_rsrc(g.a_s, 0);
+    };
+    // ids: the tile's sorted ids, either in LDS (meta buffer) or in global memory
+    auto setup_load = [&](const TileId& t, const u32* ids) __attribute__((always_inline)) {
+        const size_t sc_tile = (size_t)(g.SC / 8) * 256;           // bytes of one 32-row scale tile
+        if(STAGE == 1)
+        {
+#pragma unroll
+            for(int h = 0; h < 2; h++)
+            {
+                const size_t row = (size_t)t.e * g.N + h * I + t.nt * 128 + wave * 32;
+                wrs[h]           = make_rsrc(g.w + row * Kb, (u32)(32 * Kb));
+                wsrs[h]          = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)sc_tile);
+            }
+        }
+        else
+        {
+            const size_t row = (size_t)t.e * g.N + t.nt * 256 + wave * 64;
+            wrs[0] = wrs[1] = make_rsrc(g.w + row * Kb, (u32)(64 * Kb));
+            wsrs[0] = wsrs[1] = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)(2 * sc_tile));
+        }
+        ars  = make_rsrc(g.a_q, (u32)((size_t)g.a_rows * Kb));
+        asrs = make_rsrc(g.a_s, (u32)((size_t)g.a_rows * g.SK));
 #pragma unroll
         for(int i = 0; i < NA; i++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(asrs, LDS_PTR(sstage[s] + (wave + 4 * i) * 256), 4,
-                                                     as_off[i] + ks * 16, 0, 0, 0);
+        {
+            const int slot = wave + 4 * i;
+            int row        = 0;                      // padding rows and unused slots read row 0; never stored
+            if(slot < MT)
+            {
+                if(STAGE == 1)
+                {
+                    const u32 id  = ids[slot * 16 + dma_row];
+                    const int tok = (int)(id & 0xFFFFFFu);
+                    row           = ((int)(id >> 24) < g.topk && tok < g.T) ? tok : 0;
+                }
+                else
+                    row = t.m_blk * BM + slot * 16 + dma_row;
+            }
+            a_off[i]  = row * Kb + dma_chunk * 16;
+            as_off[i] = row * g.SK + (lane & 3) * 4;
+        }
+    };
+
+    uint8_t* const stage[2]  = {lds_a0, lds_a1};
+    uint8_t* const sstage[2] = {lds_s0, lds_s1};
+    // activation tile + scales of K-group ks -> LDS stage s.  Lane (r, kb) fetches 16 B of row r, so the
+    // 1 KB block of a (row group, K-step) lands in MFMA operand order; 5*NA VMEM ops per wave.
+    const u32 lds_a[2] = {lds_addr_of(lds_a0 + wave * 1024), lds_addr_of(lds_a1 + wave * 1024)};
+    const u32 lds_s[2] = {lds_addr_of(lds_s0 + wave * 256), lds_addr_of(lds_s1 + wave * 256)};
+    auto dma_group = [&](auto S, int ks) __attribute__((always_inline)) {
+        constexpr int s = decltype(S)::value;
+        static_for<NA>([&](auto II) __attribute__((always_inline)) {
+            constexpr int i = decltype(II)::value;
+            static_for<4>([&](auto U) __attribute__((always_inline)) {
+                constexpr int u = decltype(U)::value;
+                vm_dma_b128<u * 64, (u * SLOTS + 4 * i) * 1024>(a_off[i], ars, ks * 256, lds_a[s]);
+            });
+            vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, ks * 16, lds_s[s]);
+        });
+    };
+    v4i wf[4][4];
+    int w_sc[2][4];
+    // per-lane offsets of the wave's row groups inside wrs[] / of its scale dwords inside wsrs[]
+    const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1 (+32*Kb for stage 2, h = 1)
+    const int w_half     = (STAGE == 2) ? 32 * Kb : 0;
+    const int ws_half    = (STAGE == 2) ? (g.SC / 8) * 256 : 0;
+    auto load_wscales = [&](auto S, int ks) __attribute__((always_inline)) {
+        constexpr int s = decltype(S)::value;
+#pragma unroll
+        for(int h = 0; h < 2; h++)
+#pragma unroll
+            for(int c = 0; c < 2; c++)
+                vm_load_b32<0>(w_sc[s][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], ks * 512);
+    };
+    auto load_wtiles = [&](auto U, int kt) __attribute__((always_inline)) {
+        constexpr int u = decltype(U)::value;
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            vm_load_b128<0>(wf[u][j], w_voff[j & 1] + (j >> 1) * w_half, wrs[j >> 1], kt * 1024);
     };
 
     v4f acc[4][MT];
-#pragma unroll
-    for(int j = 0; j < 4; j++)
-#pragma unroll
-        for(int mt = 0; mt < MT; mt++)
-            acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-    // ---- prologue: activation tiles of K-steps 0..2 in flight, weight tiles of K-steps 0..3, scales of group 0
-    v4i wf[4][4];
-    int w_sc[2][4];
-    dma_s(std::integral_constant<int, 0>{}, 0);
-    dma_a(std::integral_constant<int, 0>{}, 0);
-    dma_a(std::integral_constant<int, 1>{}, 1);
-    dma_a(std::integral_constant<int, 2>{}, 2);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for(int s = 0; s < 4; s++)
+    auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for(int j = 0; j < 4; j++)
-            wf[s][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrs[j], lane * 16 + s * 1024, 0, 0));
-#pragma unroll
-    for(int h = 0; h < 2; h++)
-#pragma unroll
-        for(int c = 0; c < 2; c++)
-            w_sc[0][h * 2 + c] = *(const int*)(wsptr[h] + (size_t)c * 256);
-    __builtin_amdgcn_sched_barrier(0);
-    // scales and stage 0 must have landed: younger ops = 2*NA (DMA) + 16 + 4
-    wait_vmcnt_barrier<2 * NA + 16 + 4>();
-
-    const int KS = g.K / 512;
-    auto kgroup = [&](auto P, int ks) {
-        constexpr int p = decltype(P)::value;     // parity of ks: which scale registers are live
-        static_for<4>([&](auto U) {
-            constexpr int u = decltype(U)::value;
-            const int kt    = ks * 4 + u;
-            // (1) activation tile of K-step kt+3 -> stage (u+3)%4 (last read in step kt-1)
-            dma_a(std::integral_constant<int, (u + 3) % 4>{}, kt + 3);
-            // (2) scales of the next K-group
-            if(u == 0)
-            {
-                const int kn = ks + 1 < KS ? ks + 1 : ks;
-                dma_s(std::integral_constant<int, p ^ 1>{}, kn);
-#pragma unroll
-                for(int h = 0; h < 2; h++)
-#pragma unroll
-                    for(int c = 0; c < 2; c++)
-                        w_sc[p ^ 1][h * 2 + c] = *(const int*)(wsptr[h] + (size_t)(kn * 2 + c) * 256);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // (3) MFMAs of K-step kt.  Activation scales of the whole tile first (one dword per 16-row group, the
-            //     byte of this K-step is picked by op_sel), then tile operands two reads ahead of their MFMAs.
-            int asc[MT];
 #pragma unroll
             for(int mt = 0; mt < MT; mt++)
-                asc[mt] = *(const int*)(sstage[p] + mt * 256 + lane * 4);
-            __builtin_amdgcn_sched_barrier(0);
-            v4i af[MT];
-#pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-                af[mt] = *(const v4i*)(stage[u] + mt * 1024 + lane * 16);
-#pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-            {
-                // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                acc[0][mt] = mfma_fp4<(u & 1) * 2 + 0, u>(wf[u][0], af[mt], acc[0][mt], w_sc[p][0 + (u >> 1)], asc[mt]);
-                acc[1][mt] = mfma_fp4<(u & 1) * 2 + 1, u>(wf[u][1], af[mt], acc[1][mt], w_sc[p][0 + (u >> 1)], asc[mt]);
-                acc[2][mt] = mfma_fp4<(u & 1) * 2 + 0, u>(wf[u][2], af[mt], acc[2][mt], w_sc[p][2 + (u >> 1)], asc[mt]);
-                acc[3][mt] = mfma_fp4<(u & 1) * 2 + 1, u>(wf[u][3], af[mt], acc[3][mt], w_sc[p][2 + (u >> 1)], asc[mt]);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x100, MT < 2 ? MT : 2, 0);
-#pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-            {
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-                if(mt + 2 < MT)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // (4) weight tiles of K-step kt+4 into the registers just consumed
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-                wf[u][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wrs[j], lane * 16 + (kt + 4) * 1024, 0, 0));
-            __builtin_amdgcn_sched_barrier(0);
-            // (5) the activation tile of K-step kt+1 was DMA'd in step kt-2; VMEM ops certainly issued
-            //     after it: 4 (kt-2) + NA+S(u-1)+4 (kt-1) + NA+S(u)+4 (kt), S = scale loads (u == 0 only)
-            constexpr int S = NA + 4;
-            wait_vmcnt_barrier<12 + 2 * NA + ((u == 0 || u == 1) ? S : 0)>();
-        });
+                acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
     };
-    for(int ks = 0; ks < KS; ks += 2)
-    {
-        kgroup(std::integral_constant<int, 0>{}, ks);
-        if(ks + 1 < KS)
-            kgroup(std::integral_constant<int, 1>{}, ks + 1);
-    }
 
-    // ---------------------------------------------------------------- epilogue
-    if(STAGE == 1)
-    {
-        uint16_t* out = (uint16_t*)g.out;
-#pragma unroll
-        for(int j = 0; j < 2; j++)
+    // ---------------------------------------------------------------- epilogue of one tile
+    auto epilogue = [&](const TileId& t, const u32* meta) __attribute__((always_inline)) {
+        if(STAGE == 1)
         {
-            const int ch = nt * 128 + wave * 32 + j * 16 + kb * 4;
-            float bg[4] = {0, 0, 0, 0}, bu[4] = {0, 0, 0, 0};
-            if(g.bias)
+            // lane (r, kb) holds channels j*16 + kb*4 .. +3 (j = 0, 1) of row r.  After one permlane16 swap per
+            // packed dword a lane holds 8 consecutive channels: one 16 B store, 64 B contiguous per row and wave.
+            typedef unsigned v2u __attribute__((ext_vector_type(2)));
+            uint16_t* out = (uint16_t*)g.out;
+            const int chw = t.nt * 128 + wave * 32;
+            if(g.bias)      // rare: fold the biases into the accumulators first
             {
 #pragma unroll
-                for(int i = 0; i < 4; i++)
+                for(int j = 0; j < 4; j++)
                 {
-                    bg[i] = bf16_bits_to_f32(g.bias[(size_t)e * g.N + ch + i]);
-                    bu[i] = bf16_bits_to_f32(g.bias[(size_t)e * g.N + I + ch + i]);
+                    float b[4];
+#pragma unroll
+                    for(int i = 0; i < 4; i++)
+                        b[i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4 + i]);
+#pragma unroll
+                    for(int mt = 0; mt < MT; mt++)
+#pragma unroll
+                        for(int i = 0; i < 4; i++)
+                            acc[j][mt][i] += b[i];
+                }
+            }
+            // after the swap: lane rows 0..3 hold channel offsets 0, 16, 8, 24
+            const int ch_out = chw + (kb & 1) * 16 + (kb >> 1) * 8;
+#pragma unroll
+            for(int mt = 0; mt < MT; mt++)
+            {
+                const int p   = t.m_blk * BM + mt * 16 + r;
+                const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
+                u32 d[2][2];
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                {
+                    float v[4];
+#pragma unroll
+                    for(int i = 0; i < 4; i++)
+                        v[i] = ok ? silu_f32(acc[j][mt][i]) * acc[j + 2][mt][i] : 0.f;
+                    d[j][0] = pack_bf16x2(v[0], v[1]);
+                    d[j][1] = pack_bf16x2(v[2], v[3]);
+                }
+                v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
+                v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
+                // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
+                *(uint4*)(out + (size_t)p * I + ch_out) = make_uint4(t0.x, t1.x, t0.y, t1.y);
+                __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
+            }
+        }
+        else
+        {
+            // lane (r, kb) holds channels j*16 + kb*4 .. +3 (j = 0..3) of row r.  A 4x4 transpose across the
+            // four lane rows gives every lane 16 consecutive channels: 32 B stores, 128 B contiguous per row.
+            uint16_t* out = (uint16_t*)g.out;
+            const int chw = t.nt * 256 + wave * 64;
+            if(g.bias)      // rare: fold the bias into the accumulators first
+            {
+#pragma unroll
+                for(int j = 0; j < 4; j++)
+                {
+                    float b[4];
+#pragma unroll
+                    for(int i = 0; i < 4; i++)
+                        b[i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + chw + j * 16 + kb * 4 + i]);
+#pragma unroll
+                    for(int mt = 0; mt < MT; mt++)
+#pragma unroll
+                        for(int i = 0; i < 4; i++)
+                            acc[j][mt][i] += b[i];
                 }
             }
 #pragma unroll
             for(int mt = 0; mt < MT; mt++)
             {
-                const int p  = m_blk * BM + mt * 16 + r;
-                const u32 id = g.sorted_ids[p];
-                const bool ok = (int)(id >> 24) < g.topk;
-                float v[4];
+                const u32 id   = meta[mt * 16 + r];
+                const float rw = __builtin_bit_cast(float, meta[MPAD + mt * 16 + r]);
+                const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
+                const bool ok = slot < g.topk && tok < g.T;
+                u32 lo[4], hi[4];
 #pragma unroll
-                for(int i = 0; i < 4; i++)
-                    v[i] = ok ? silu_f32(acc[j][mt][i] + bg[i]) * (acc[j + 2][mt][i] + bu[i]) : 0.f;
-                uint2 o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-                *(uint2*)(out + (size_t)p * I + ch) = o;
+                for(int j = 0; j < 4; j++)
+                {
+                    lo[j] = pack_bf16x2(acc[j][mt][0] * rw, acc[j][mt][1] * rw);
+                    hi[j] = pack_bf16x2(acc[j][mt][2] * rw, acc[j][mt][3] * rw);
+                }
+                transpose4x4_rows(lo);
+                transpose4x4_rows(hi);
+                // lane row q now holds channels q*16 + c*4 .. +3 in (lo[c], hi[c])
+                if(ok)
+                {
+                    uint4* dst = (uint4*)(out + ((size_t)tok * g.topk + slot) * g.N + chw + kb * 16);
+                    dst[0]     = make_uint4(lo[0], hi[0], lo[1], hi[1]);
+                    dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
+                }
+                __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
             }
         }
-    }
-    else
+    };
+
+    // ---------------------------------------------------------------- pipeline
+#ifdef PYHIP_GEMM_DEBUG
+    unsigned long long tacc[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, t0 = wall_clock64(), t1;
+    const unsigned long long c_start = __builtin_readcyclecounter(), w_start = t0;
+#define TICK(i) do { t1 = wall_clock64(); tacc[i] += t1 - t0; t0 = t1; } while(0)
+#else
+#define TICK(i)
+#endif
+    TileId cur, nxt;
+    decode(cur);
+    if(!cur.valid)
     {
-        uint16_t* out = (uint16_t*)g.out;
-#pragma unroll
-        for(int mt = 0; mt < MT; mt++)
-        {
-            const int p  = m_blk * BM + mt * 16 + r;
-            const u32 id = g.sorted_ids[p];
-            const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
-            if(slot >= g.topk || tok >= g.T)
-                continue;
-            const float rw = g.sorted_w[p];
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-            {
-                const int ch = nt * 256 + wave * 64 + j * 16 + kb * 4;
-                float b[4] = {0, 0, 0, 0};
-                if(g.bias)
-#pragma unroll
-                    for(int i = 0; i < 4; i++)
-                        b[i] = bf16_bits_to_f32(g.bias[(size_t)e * g.N + ch + i]);
-                uint2 o = make_uint2(pack_bf16x2((acc[j][mt][0] + b[0]) * rw, (acc[j][mt][1] + b[1]) * rw),
-                                     pack_bf16x2((acc[j][mt][2] + b[2]) * rw, (acc[j][mt][3] + b[3]) * rw));
-                *(uint2*)(out + ((size_t)tok * g.topk + slot) * g.N + ch) = o;
-            }
-        }
+        if(persistent && tid == 0 && rounds_total)   // no tile at all: credit every round at once
+            __hip_atomic_fetch_add(rendezvous, rounds_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
     }
+    int mb = 0;                                   // meta buffer of the current tile (ring of 3)
+    setup_load(cur, g.sorted_ids + (size_t)cur.m_blk * BM);
+    // prologue, in the K-group's issue order: this tile's ids/weights, activation K-group 0, weight scales of
+    // group 0, weight tiles of K-steps 0..3
+    dma_meta(cur, 0, true);
+    dma_group(std::integral_constant<int, 0>{}, 0);
+    load_wscales(std::integral_constant<int, 0>{}, 0);
+    static_for<4>([&](auto U) __attribute__((always_inline)) { load_wtiles(U, decltype(U)::value); });
+    wait_vmcnt_barrier<16>();         // everything older than the weight tiles has landed
+    decode(nxt);                      // (without a schedule there is no next tile)
+    zero_acc();
+    int ks = 0;
+    TICK(0);                          // start-up
+
+    // one K-group; returns false when the workgroup has no more work
+    auto kgroup = [&](auto P) __attribute__((always_inline)) -> bool {
+        constexpr int p = decltype(P)::value;     // parity of the global K-group count: LDS stage / scale registers
+        const bool last     = ks == KS - 1;
+        const int kpre      = last ? 0 : ks + 1;  // K-group that is prefetched now (of the next tile when last)
+        const int mb_nxt    = mb == 2 ? 0 : mb + 1;
+        TICK(1);                      // loop overhead since the last tick
+        // (0) first K-group of a tile: ids/weights of the NEXT tile into the meta ring (two tiles ahead of the
+        //     slot any wave can still be reading in its epilogue)
+        // (1) descriptors of what this K-group prefetches: the next K-group of this tile, or K-group 0 of the
+        //     next tile (into the other LDS stage, whose readers left at the last barrier)
+        if(last)
+        {
+            if(nxt.valid)
+                setup_load(nxt, lds_meta[mb_nxt]);
+            else
+                setup_null();
+        }
+#ifdef PYHIP_GEMM_DEBUG
+        if(g.dbg & 3) setup_null();
+#endif
+        const bool meta_on = ks == 0 && nxt.valid;
+        const v4i rid = make_rsrc(g.sorted_ids + (size_t)nxt.m_blk * BM, BM * 4);
+        const v4i rwt = make_rsrc(g.sorted_w + (size_t)nxt.m_blk * BM, BM * 4);
+        // prefetch operation K of this K-group (0 <= K < NPF)
+        auto prefetch_op = [&](auto KK) __attribute__((always_inline)) {
+            constexpr int k = decltype(KK)::value;
+            if constexpr(k < NM)
+            {
+                // ids/weights of the NEXT tile into the meta ring (first K-group of a tile only; two tiles ahead
+                // of the slot any wave can still be reading in its epilogue)
+                const int o     = wave + 4 * k;           // op index: [0, NID) ids, [NID, 2*NID) weights, beyond: nothing
+                const bool wts  = o >= NID;
+                const int oo    = wts ? o - NID : o;
+                const bool real = meta_on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
+                // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
+                const v4i rs    = real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0);
+                const u32 dst   = real ? lds_addr_of(&lds_meta[mb_nxt][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy);
+                vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
+            }
+            else if constexpr(k < NM + 5 * NA)
+            {
+                constexpr int i = (k - NM) / 5, sub = (k - NM) % 5;
+                if constexpr(sub < 4)
+                    vm_dma_b128<sub * 64, (sub * SLOTS + 4 * i) * 1024>(a_off[i], ars, kpre * 256, lds_a[p ^ 1]);
+                else
+                    vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, kpre * 16, lds_s[p ^ 1]);
+            }
+            else
+            {
+                constexpr int h = (k - NM - 5 * NA) / 2, c = (k - NM - 5 * NA) % 2;
+                vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], kpre * 512);
+            }
+        };
+        TICK(6);                      // tile bookkeeping
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<4>([&](auto U) __attribute__((always_inline)) {
+            constexpr int u = decltype(U)::value;
+            // (3) MFMAs of K-step 4*ks + u, tile operands two reads ahead of their MFMAs.  The weight tiles of
+            //     this K-step (and, at u = 0, the weight scales) were requested one K-group ago.
+            constexpr int YOUNGER = u == 0 ? 12 : 12 + NPF;
+            wait_vm_tiles<YOUNGER>(wf[u][0], wf[u][1], wf[u][2], wf[u][3]);
+            if(u == 0)
+                wait_vm_scales<YOUNGER>(w_sc[p][0], w_sc[p][1], w_sc[p][2], w_sc[p][3]);
+            // activation operand and its scale dword (one per 16-row group and K-group, op_sel picks this K-step's
+            // byte) are read one row group ahead of the MFMAs that consume them
+            v4i af  = *(const v4i*)(stage[p] + (u * SLOTS) * 1024 + rd_a);
+            int asc = *(const int*)(sstage[p] + rd_s);
+            static_for<MT>([&](auto M) __attribute__((always_inline)) {
+                constexpr int mt = decltype(M)::value;
+                v4i af_n  = af;
+                int asc_n = asc;
+                if constexpr(mt + 1 < MT)
+                {
+                    af_n  = *(const v4i*)(stage[p] + (u * SLOTS + mt + 1) * 1024 + rd_a);
+                    asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#ifdef PYHIP_GEMM_DEBUG
+                if(!(g.dbg & 4))
+#endif
+                {
+                // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
+                mfma_fp4<(u & 1) * 2 + 0, u>(acc[0][mt], wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
+                mfma_fp4<(u & 1) * 2 + 1, u>(acc[1][mt], wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
+                mfma_fp4<(u & 1) * 2 + 0, u>(acc[2][mt], wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
+                mfma_fp4<(u & 1) * 2 + 1, u>(acc[3][mt], wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
+                }
+                // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
+                // issue overlaps the matrix pipeline instead of preceding it
+                if constexpr(u == 0)
+                    static_for<PPM>([&](auto Q) __attribute__((always_inline)) {
+                        constexpr int k = mt * PPM + decltype(Q)::value;
+                        if constexpr(k < NPF)
+                            prefetch_op(std::integral_constant<int, k>{});
+                    });
+                __builtin_amdgcn_sched_barrier(0);
+                af  = af_n;
+                asc = asc_n;
+            });
+            __builtin_amdgcn_sched_barrier(0);
+            // (4) weight tiles of the same K-step of the prefetched K-group into the registers just consumed
+            load_wtiles(U, kpre * 4 + u);
+            __builtin_amdgcn_sched_barrier(0);
+            TICK(7 + u);
+        });
+        // (5) the 16 weight loads above are the only VMEM ops younger than this group's DMAs
+        wait_vmcnt_barrier<16>();
+        TICK(2);                      // wait + barrier
+        ks++;
+        if(last)
+        {
+            // the last MFMAs were issued from assembly: give their results the documented distance to the
+            // first VALU read
+            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+            epilogue(cur, lds_meta[mb]);
+            TICK(3);
+#ifdef PYHIP_GEMM_DEBUG
+            tacc[5] += 1;
+#endif
+            if(!nxt.valid)
+            {
+                if(persistent && tid == 0 && rounds_total > rounds_done)   // leaving: credit the rounds not joined
+                    __hip_atomic_fetch_add(rendezvous, rounds_total - rounds_done, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                return false;
+            }
+            cur = nxt;
+            mb  = mb_nxt;
+            ks  = 0;
+            zero_acc();
+            decode(nxt);
+            meet();
+            TICK(4);
+        }
+        return true;
+    };
+    for(;;)
+    {
+        if(!kgroup(std::integral_constant<int, 0>{}))
+            break;
+        if(!kgroup(std::integral_constant<int, 1>{}))
+            break;
+    }
+#ifdef PYHIP_GEMM_DEBUG
+    if(g.dbg_t && threadIdx.x == 0)
+    {
+        tacc[1]  = __builtin_readcyclecounter() - c_start;   // shader clocks over the kernel
+        tacc[11] = wall_clock64() - w_start;                 // 100 MHz ticks over the kernel
+        for(int i = 0; i < 12; i++)
+            g.dbg_t[blockIdx.x * 12 + i] = tacc[i];
+    }
+#endif
 #endif
 }
 
 template <int STAGE>
-static int launch_gemm(const GemmArgs& g, int block_m, hipStream_t stream)
+static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
 {
-    dim3 grid((unsigned)(g.n_tiles * g.n_blk)), block(GEMM_THREADS);
+#ifdef PYHIP_GEMM_DEBUG
+    g.dbg = getenv("PYHIP_DBG") ? atoi(getenv("PYHIP_DBG")) : 0;
+    g.dbg_t = getenv("PYHIP_DBG_T") ? (unsigned long long*)strtoull(getenv("PYHIP_DBG_T"), nullptr, 0) : nullptr;
+#endif
+    unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
+    if(g.K < 1024)
+        g.sched = nullptr;   // a single K-group per tile: no room to prefetch across tiles, one tile per workgroup
+    if(g.sched)
+    {
+        // persistent: fill every CU at the kernel's occupancy (2 workgroups per CU up to 128 rows, else 1)
+        int dev = 0, cus = 256;
+        if(hipGetDevice(&dev) == hipSuccess)
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
+        nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
+    }
+    dim3 grid(nwg), block(GEMM_THREADS);
     switch(block_m)
     {
     case 16: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 1>), grid, block, 0, stream, g); break;
@@ -351,9 +729,9 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 
 extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1,
                                      const uint8_t* w1_scale, const void* bias1_bf16, const uint32_t* sorted_ids,
-                                     const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* a2_bf16,
-                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, hipStream_t stream)
+                                     const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
+                                     const uint32_t* schedule, void* a2_bf16, int tokens, int topk, int experts,
+                                     int hidden, int inter, int block_m, int64_t n_blk, hipStream_t stream)
 {
     int rc = check_common("moe_gemm1", a_q, a_scale, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                           a2_bf16, hidden, block_m, n_blk, tokens);
@@ -366,7 +744,7 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
     GemmArgs g;
     g.a_q = a_q; g.a_s = a_scale; g.w = w1; g.w_s = w1_scale; g.bias = (const uint16_t*)bias1_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
-    g.out = a2_bf16;
+    g.out = a2_bf16; g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
     g.SK = (hidden + 511) / 512 * 16;
     g.SC = (hidden / 32 + 7) / 8 * 8;
@@ -377,9 +755,9 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
 extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2,
                                      const uint8_t* w2_scale, const void* bias2_bf16, const uint32_t* sorted_ids,
                                      const float* sorted_weights, const uint32_t* sorted_expert_ids,
-                                     const uint32_t* num_valid_ids, void* out3_bf16, int tokens, int topk,
-                                     int experts, int hidden, int inter, int block_m, int64_t n_blk,
-                                     hipStream_t stream)
+                                     const uint32_t* num_valid_ids, const uint32_t* schedule, void* out3_bf16,
+                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                     int64_t n_blk, hipStream_t stream)
 {
     int rc = check_common("moe_gemm2", a2_q, a2_scale, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                           out3_bf16, inter, block_m, n_blk, n_blk * block_m);
@@ -393,7 +771,7 @@ extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scal
     GemmArgs g;
     g.a_q = a2_q; g.a_s = a2_scale; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
-    g.num_valid = num_valid_ids; g.out = out3_bf16;
+    g.num_valid = num_valid_ids; g.out = out3_bf16; g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = inter; g.N = hidden;
     g.SK = (inter + 511) / 512 * 16;
     g.SC = (inter / 32 + 7) / 8 * 8;

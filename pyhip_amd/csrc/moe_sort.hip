@@ -31,7 +31,8 @@ struct SortArgs
     float* sorted_w;
     u32* sorted_e;
     u32* num_valid;
-    u32* ws;                   // workspace: hist[G][E], then per-expert offset[E], total[E], local_id[E]
+    u32* ws;                   // workspace: hist[G][E], then per-expert offset[E]
+    u32* sched;                // optional tile schedule for the grouped GEMMs (see write_schedule) or null
     int T_all, k, E, Bm, n_blk, G;
 };
 
@@ -196,6 +197,51 @@ __device__ __forceinline__ void fill_outputs(const SortArgs& a, const u32* tot, 
     }
 }
 
+// Tile schedule for the persistent grouped GEMMs.  Experts are dealt to the 8 XCDs (expert e -> XCD e % 8)
+// so that all row blocks and weight tiles of an expert meet in one L2.  Layout (u32 words), EX = E/8 + 2:
+//   sched[x*EX + i], i = 0..EX-1 : number of row blocks owned by the first i experts of XCD x
+//                                  (experts x, x+8, x+16, ...; entries past the last expert repeat the total)
+//   sched[8*EX + e]              : first row block of expert e
+//   sched[8*EX + E + e]          : local id of expert e (its index among the unmasked experts)
+//   sched[8*EX + 2E + i], i < 16 : zeroed; per-XCD arrival counters of the two grouped GEMMs
+// One workgroup; uses the first 8 waves.
+__device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot, const u32* off, const u32* lid)
+{
+    if(!a.sched)
+        return;
+    const int EX   = a.E / 8 + 2;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    if(wave < 8)
+    {
+        u32 run = 0;
+        for(int i0 = 0; i0 < EX; i0 += WAVE)
+        {
+            const int i = i0 + lane;
+            const int e = wave + 8 * i;
+            u32 nb      = 0;
+            if(i < EX && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0))
+                nb = (tot[e] + a.Bm - 1) / a.Bm;
+            u32 sc = nb;
+            for(int d = 1; d < WAVE; d <<= 1)
+            {
+                u32 t = __shfl_up(sc, d);
+                if(lane >= d)
+                    sc += t;
+            }
+            if(i < EX)
+                a.sched[wave * EX + i] = run + sc - nb;
+            run += __shfl(sc, WAVE - 1);
+        }
+    }
+    for(int e = threadIdx.x; e < a.E; e += blockDim.x)
+    {
+        a.sched[8 * EX + e]       = off[e] / a.Bm;
+        a.sched[8 * EX + a.E + e] = lid[e];
+    }
+    if(threadIdx.x < 16)
+        a.sched[8 * EX + 2 * a.E + threadIdx.x] = 0;
+}
+
 // ---------------------------------------------------------------------------------------------
 // single workgroup: everything in one launch (decode-sized inputs)
 // LDS: whist[SMALL_WAVES][E] | tot[E] | off[E] | lid[E] | scratch[2*SMALL_WAVES]
@@ -233,6 +279,7 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kerne
     __syncthreads();
     u32 padded_total = expert_offsets(a, tot, off, lid, scratch);
     fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+    write_schedule(a, tot, off, lid);
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         for(int w = 0; w < SMALL_WAVES; w++)
             whist[w * a.E + e] += off[e];
@@ -286,6 +333,7 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         g_off[e] = off[e];
     fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+    write_schedule(a, tot, off, lid);
 }
 
 // launch 3 of 3: scatter.  LDS: whist[SORT_WAVES][E]
@@ -353,11 +401,13 @@ extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, i
     return ((int64_t)sort_groups(pairs) + 1) * experts * 4 + 256;
 }
 
+extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 8ll * (experts / 8 + 2) + 2ll * experts + 16; }
+
 extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
                                  int experts, int block_size, const int32_t* expert_mask,
                                  const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
-                                 uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, void* moe_out,
-                                 int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
+                                 uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
+                                 void* moe_out, int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
                                  hipStream_t stream)
 {
     PYHIP_REQUIRE(topk_ids && topk_weights && sorted_ids && sorted_weights && sorted_expert_ids && num_valid_ids,
@@ -382,6 +432,7 @@ extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weig
     a.sorted_e      = sorted_expert_ids;
     a.num_valid     = num_valid_ids;
     a.ws            = (u32*)workspace;
+    a.sched         = schedule;
     a.T_all         = tokens;
     a.k             = topk;
     a.E             = experts;

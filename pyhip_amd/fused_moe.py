@@ -114,9 +114,9 @@ def fused_moe(
     topk_weight = topk_weight.to(torch.float32).contiguous()
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
     ev = _mark("start")
-    sorted_ids, sorted_w, sorted_e, num_valid, _ = moe_sorting(
+    sorted_ids, sorted_w, sorted_e, num_valid, _, sched = moe_sorting(
         topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
-        moe_sorting_dispatch_policy, alloc_moe_out=False)
+        moe_sorting_dispatch_policy, alloc_moe_out=False, return_schedule=True)
     ev = _mark("sort", ev)
     n_blk = sorted_e.numel()
     stream = _lib.current_stream()
@@ -133,7 +133,8 @@ def fused_moe(
     ev = _mark("quant1", ev)
     rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                    _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
-                                   _lib.dptr(num_valid), _lib.dptr(a2), T, k, E, H, I, bm, n_blk, stream)
+                                   _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), T, k, global_E, H, I, bm,
+                                   n_blk, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
     a2_q, a2_s = act_quant_mxfp4(a2, rows_limit=num_valid)
@@ -143,8 +144,8 @@ def fused_moe(
     ev = _mark("quant2", ev)
     rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
                                    _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
-                                   _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(out3),
-                                   T, k, E, H, I, bm, n_blk, stream)
+                                   _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
+                                   T, k, global_E, H, I, bm, n_blk, stream)
     _lib.check(rc, "moe_gemm2_mxfp4")
     ev = _mark("gemm2", ev)
     out = torch.empty(T, H, dtype=out_dtype, device=dev)

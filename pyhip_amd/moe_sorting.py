@@ -13,7 +13,8 @@ def max_blocks(num_pairs, num_experts, block_size):
 
 
 def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, block_size=32,
-                expert_mask=None, num_local_tokens=None, dispatch_policy=0, *, alloc_moe_out=True):
+                expert_mask=None, num_local_tokens=None, dispatch_policy=0, *, alloc_moe_out=True,
+                return_schedule=False):
     """-> (sorted_ids u32 [n_blk*Bm] viewed as int32, sorted_weights f32, sorted_expert_ids int32 [n_blk],
     num_valid_ids int32 [2], moe_out [T, model_dim] zero-filled)
 
@@ -33,6 +34,8 @@ def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, bl
     sorted_e = torch.empty(n_blk, dtype=torch.int32, device=dev)
     num_valid = torch.empty(2, dtype=torch.int32, device=dev)
     moe_out = torch.empty(T, model_dim, dtype=moebuf_dtype, device=dev) if alloc_moe_out else None
+    sched = torch.empty(lib.pyhip_moe_schedule_words(num_experts), dtype=torch.int32, device=dev) \
+        if return_schedule else None
     ws_bytes = lib.pyhip_moe_sorting_workspace_bytes(T, k, num_experts)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if expert_mask is not None:
@@ -43,8 +46,10 @@ def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, bl
     rc = lib.pyhip_moe_sorting(
         _lib.dptr(topk_ids), _lib.dptr(topk_weights), T, k, num_experts, block_size,
         _lib.dptr(expert_mask), _lib.dptr(num_local_tokens),
-        _lib.dptr(sorted_ids), _lib.dptr(sorted_w), _lib.dptr(sorted_e), _lib.dptr(num_valid),
+        _lib.dptr(sorted_ids), _lib.dptr(sorted_w), _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched),
         _lib.dptr(moe_out), 0 if moe_out is None else moe_out.numel() * moe_out.element_size(),
         _lib.dptr(ws), ws_bytes, _lib.current_stream())
     _lib.check(rc, "moe_sorting")
+    if return_schedule:
+        return sorted_ids, sorted_w, sorted_e, num_valid, moe_out, sched
     return sorted_ids, sorted_w, sorted_e, num_valid, moe_out

@@ -34,20 +34,21 @@ def test_size_helpers():
     assert lib.pyhip_moe_act_scale_stride(7168) == 224 and lib.pyhip_moe_act_scale_stride(1024) == 32
     assert lib.pyhip_moe_act_scale_stride(2880) == 96
     assert lib.pyhip_moe_sorting_workspace_bytes(16, 8, 256) >= 0
+    assert lib.pyhip_moe_schedule_words(256) == 8 * 34 + 512 + 16
 
 
 def test_argument_errors_are_reported():
     lib = _lib.load()
-    rc = lib.pyhip_moe_sorting(None, None, 4, 2, 8, 16, None, None, None, None, None, None, None, 0, None, 0, None)
+    rc = lib.pyhip_moe_sorting(None, None, 4, 2, 8, 16, None, None, None, None, None, None, None, None, 0, None, 0, None)
     assert rc == 1
     with pytest.raises(_lib.PyhipError, match="null pointer"):
         _lib.check(rc, "moe_sorting")
     one = ctypes.c_void_p(16)
     rc = lib.pyhip_moe_act_quant_mxfp4(one, 40, 4, 40, one, one, None, None)
     assert rc == 1 and b"multiple of 32" in lib.pyhip_moe_last_error()
-    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, one, 4, 2, 8, 1000, 512, 16, 4, None)
+    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, 4, 2, 8, 1000, 512, 16, 4, None)
     assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
-    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, one, 4, 2, 8, 1024, 512, 48, 4, None)
+    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 48, 4, None)
     assert rc == 1 and b"block_m" in lib.pyhip_moe_last_error()
 
 
