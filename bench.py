@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--decode-tokens", type=int, default=16)
     ap.add_argument("--block-m", type=int, default=0)
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="target size of the CPU sample; 0 = skip")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
     return ap.parse_args()
 
 
@@ -119,6 +121,14 @@ def main():
     torch.cuda.synchronize()
     main_res = run_config(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m)
     dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
+
+    if a.calibrate_copy:
+        src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     w = main_res["work"]
     tflops = w["flops"] / (main_res["ms"] * 1e-3) / 1e12

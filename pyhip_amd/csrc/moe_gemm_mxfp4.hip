@@ -148,7 +148,7 @@ struct TileId
 // a tile boundary needs (schedule tables, sorted ids, routing weights) is read from LDS, so no wait on the
 // vector-memory counter ever covers the prefetches in flight.
 template <int STAGE, int MT>
-__global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp4_kernel(GemmArgs g)
+__global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     constexpr int BM    = MT * 16;
@@ -193,8 +193,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
     const u32 qstride     = gridDim.x >> 3;
     u32 q                 = blockIdx.x >> 3;
     int ei                = 0;                        // cursor into this XCD's expert list (q only grows)
-    const u32 wgs_on_xcd  = gridDim.x >> 3;
-    u32 rounds_total      = 0;                        // rounds this XCD's tile list needs
     if(persistent)
     {
         for(int i = tid; i < EX; i += GEMM_THREADS)
@@ -205,33 +203,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
             lds_lid[i]   = e < g.E ? g.sched[8 * EX + g.E + e] : 0u;
         }
         __syncthreads();
-        rounds_total = (lds_pre[EX - 1] * (u32)g.n_tiles + wgs_on_xcd - 1) / wgs_on_xcd;
     }
     auto uni = [](u32 v) __attribute__((always_inline)) { return (u32)__builtin_amdgcn_readfirstlane((int)v); };
-    // ---- per-tile rendezvous of the workgroups of one XCD.  Tiles that share a weight tile (the row blocks of
-    // one expert) or an activation tile sit next to each other in the XCD's list, so they are in flight in the
-    // same round; meeting once per round keeps the workgroups within a K-group or two of each other, which is
-    // what lets the second reader of a line find it in the XCD's L2 (4 MB hold only a few microseconds of
-    // traffic).  The counter lives in the schedule buffer and is zeroed by the sort.  The wait is bounded: a
-    // missing workgroup costs time, never a hang.
-    u32* const rendezvous = persistent ? const_cast<u32*>(g.sched) + 8 * EX + 2 * g.E + (STAGE - 1) * 8 + xcd : nullptr;
-    u32 rounds_done       = 0;
-    auto meet = [&]() __attribute__((always_inline)) {
-        if(!persistent)
-            return;
-        rounds_done++;
-        if(tid == 0)
-        {
-            __hip_atomic_fetch_add(rendezvous, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const u32 target = rounds_done * wgs_on_xcd;
-            for(int spin = 0; spin < 4000; spin++)
-            {
-                if(__hip_atomic_load(rendezvous, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target)
-                    break;
-                __builtin_amdgcn_s_sleep(8);
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    auto uni4 = [](v4i v) __attribute__((always_inline)) {
+        return (v4i){__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y),
+                     __builtin_amdgcn_readfirstlane(v.z), __builtin_amdgcn_readfirstlane(v.w)};
     };
     auto decode = [&](TileId& t) __attribute__((always_inline)) {
         t.valid = false;
@@ -275,8 +251,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
             const int oo    = wts ? o - NID : o;
             const bool real = on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
             // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
-            const v4i rs    = real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0);
-            const u32 dst   = real ? lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy);
+            const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
+            const u32 dst   = uni(real ? lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
             vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
         }
     };
@@ -492,7 +468,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
     };
 
     // ---------------------------------------------------------------- pipeline
-#ifdef PYHIP_GEMM_DEBUG
+#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
     unsigned long long tacc[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, t0 = wall_clock64(), t1;
     const unsigned long long c_start = __builtin_readcyclecounter(), w_start = t0;
 #define TICK(i) do { t1 = wall_clock64(); tacc[i] += t1 - t0; t0 = t1; } while(0)
@@ -502,11 +478,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
     TileId cur, nxt;
     decode(cur);
     if(!cur.valid)
-    {
-        if(persistent && tid == 0 && rounds_total)   // no tile at all: credit every round at once
-            __hip_atomic_fetch_add(rendezvous, rounds_total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
-    }
     int mb = 0;                                   // meta buffer of the current tile (ring of 3)
     setup_load(cur, g.sorted_ids + (size_t)cur.m_blk * BM);
     // prologue, in the K-group's issue order: this tile's ids/weights, activation K-group 0, weight scales of
@@ -557,8 +529,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
                 const int oo    = wts ? o - NID : o;
                 const bool real = meta_on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
                 // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
-                const v4i rs    = real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0);
-                const u32 dst   = real ? lds_addr_of(&lds_meta[mb_nxt][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy);
+                const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
+                const u32 dst   = uni(real ? lds_addr_of(&lds_meta[mb_nxt][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
                 vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
             }
             else if constexpr(k < NM + 5 * NA)
@@ -638,22 +610,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             epilogue(cur, lds_meta[mb]);
             TICK(3);
-#ifdef PYHIP_GEMM_DEBUG
+#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
             tacc[5] += 1;
 #endif
             if(!nxt.valid)
-            {
-                if(persistent && tid == 0 && rounds_total > rounds_done)   // leaving: credit the rounds not joined
-                    __hip_atomic_fetch_add(rendezvous, rounds_total - rounds_done, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
                 return false;
-            }
             cur = nxt;
             mb  = mb_nxt;
             ks  = 0;
             zero_acc();
             decode(nxt);
-            meet();
             TICK(4);
         }
         return true;
@@ -665,7 +631,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT <= 8 ? 2 : 1)) moe_gemm_mxfp
         if(!kgroup(std::integral_constant<int, 1>{}))
             break;
     }
-#ifdef PYHIP_GEMM_DEBUG
+#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
     if(g.dbg_t && threadIdx.x == 0)
     {
         tacc[1]  = __builtin_readcyclecounter() - c_start;   // shader clocks over the kernel
@@ -689,11 +655,11 @@ static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
         g.sched = nullptr;   // a single K-group per tile: no room to prefetch across tiles, one tile per workgroup
     if(g.sched)
     {
-        // persistent: fill every CU at the kernel's occupancy (2 workgroups per CU up to 128 rows, else 1)
+        // persistent: fill every CU at the kernel's occupancy (2 workgroups per CU)
         int dev = 0, cus = 256;
         if(hipGetDevice(&dev) == hipSuccess)
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
+        unsigned resident = (unsigned)cus * 2u / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
     dim3 grid(nwg), block(GEMM_THREADS);
@@ -703,8 +669,7 @@ static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
     case 32: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 2>), grid, block, 0, stream, g); break;
     case 64: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 4>), grid, block, 0, stream, g); break;
     case 128: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 8>), grid, block, 0, stream, g); break;
-    case 256: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 16>), grid, block, 0, stream, g); break;
-    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256}", block_m); return PYHIP_ERR_INVALID;
+    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128}", block_m); return PYHIP_ERR_INVALID;
     }
     PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel");
     return PYHIP_OK;
@@ -716,8 +681,8 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 {
     PYHIP_REQUIRE(a_q && a_s && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
     PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
-    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256,
-                  "%s: block_m=%d not in {16,32,64,128,256}", name, block_m);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128,
+                  "%s: block_m=%d not in {16,32,64,128}", name, block_m);
     PYHIP_REQUIRE(n_blk >= 0 && n_blk < (1 << 24), "%s: n_blk=%lld", name, (long long)n_blk);
     PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < (1ll << 32),
                   "%s: activation matrix of %lld rows x %d exceeds the 4 GiB buffer range", name, (long long)a_rows, K);

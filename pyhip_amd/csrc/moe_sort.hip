@@ -203,7 +203,6 @@ __device__ __forceinline__ void fill_outputs(const SortArgs& a, const u32* tot, 
 //                                  (experts x, x+8, x+16, ...; entries past the last expert repeat the total)
 //   sched[8*EX + e]              : first row block of expert e
 //   sched[8*EX + E + e]          : local id of expert e (its index among the unmasked experts)
-//   sched[8*EX + 2E + i], i < 16 : zeroed; per-XCD arrival counters of the two grouped GEMMs
 // One workgroup; uses the first 8 waves.
 __device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot, const u32* off, const u32* lid)
 {
@@ -238,8 +237,6 @@ __device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot
         a.sched[8 * EX + e]       = off[e] / a.Bm;
         a.sched[8 * EX + a.E + e] = lid[e];
     }
-    if(threadIdx.x < 16)
-        a.sched[8 * EX + 2 * a.E + threadIdx.x] = 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -401,7 +398,7 @@ extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, i
     return ((int64_t)sort_groups(pairs) + 1) * experts * 4 + 256;
 }
 
-extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 8ll * (experts / 8 + 2) + 2ll * experts + 16; }
+extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 8ll * (experts / 8 + 2) + 2ll * experts; }
 
 extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
                                  int experts, int block_size, const int32_t* expert_mask,
