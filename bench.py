@@ -41,8 +41,10 @@ def parse():
 def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m):
     from pyhip_amd import workloads
     hidden, topk_w, topk_ids = workloads.make_inputs(shape, tokens)
+    if W["hidden_pad"]:      # padded shapes (gpt-oss): activations at the padded width, as the reference passes them
+        hidden = torch.nn.functional.pad(hidden, (0, W["hidden_pad"]))
     kw = dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
-              block_size_M=block_m or None)
+              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"])
     for _ in range(warmup):
         out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, **kw)
     torch.cuda.synchronize()
@@ -79,6 +81,8 @@ def cpu_baseline(torch, W, shape, res, budget_s):
     from pyhip_amd import mxfp4, workloads
     cfg = workloads.SHAPES[shape]
     E, H, I, k = cfg["E"], cfg["H"], cfg["I"], cfg["k"]
+    flop_dims = I * H                                # FLOPs are counted at the true sizes
+    H, I = H + W["hidden_pad"], I + W["intermediate_pad"]
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     w1q = LazyExperts(lambda e: mxfp4.deshuffle_weight(W["w1"][e]).cpu().numpy(), (E, 2 * I, H // 2))
@@ -100,7 +104,7 @@ def cpu_baseline(torch, W, shape, res, budget_s):
         pairs += int((ids == e).sum())
         if t_total >= budget_s:
             break
-    flops = 6.0 * pairs * I * H
+    flops = 6.0 * pairs * flop_dims
     return dict(value=flops / t_total / 1e12, unit="TFLOP/s", cores=threads, kind="port",
                 sample="%d of %d hit experts (%d of %d token-expert pairs) of the %s T=%d layer, %.1f s; "
                        "includes per-expert weight dequantisation and the quantisation of all activations"

@@ -82,7 +82,6 @@ def fused_moe(
     assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
     assert not doweight_stage1
     assert a1_scale is None and a2_scale is None, "activations are quantised dynamically"
-    assert hidden_pad == 0 and intermediate_pad == 0
     assert splitk == 0
     assert w1_scale is not None and w2_scale is not None
     assert hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2
@@ -90,6 +89,14 @@ def fused_moe(
     assert out_dtype in (torch.bfloat16, torch.float32)
 
     w1u, w2u, w1s, w2s = _as_u8(w1), _as_u8(w2), _as_u8(w1_scale), _as_u8(w2_scale)
+    # hidden_pad / intermediate_pad: the weights arrive zero-padded to the kernels' tile multiples and the last
+    # hidden_pad (intermediate_pad) channels are padding.  The activations may come at the padded width (the
+    # reference's convention) or at the true width, in which case they are widened here and the result is
+    # returned at the true width.
+    assert 0 <= hidden_pad < w1u.shape[2] * 2 and 0 <= intermediate_pad < w1u.shape[1] // 2
+    narrow = hidden_pad > 0 and hidden_states.shape[1] == w1u.shape[2] * 2 - hidden_pad
+    if narrow:
+        hidden_states = torch.nn.functional.pad(hidden_states, (0, hidden_pad))
     T, H = hidden_states.shape
     k = topk_ids.shape[1]
     E, N1, Hb = w1u.shape
@@ -153,6 +160,8 @@ def fused_moe(
                                    1 if out_dtype == torch.float32 else 0, None, stream)
     _lib.check(rc, "moe_topk_reduce")
     _mark("reduce", ev)
+    if narrow:
+        out = out[:, : H - hidden_pad]
     if return_parts:
         return out, dict(sorted_ids=sorted_ids, sorted_weights=sorted_w, sorted_expert_ids=sorted_e,
                          num_valid_ids=num_valid, a1_q=a1_q, a1_s=a1_s, a2=a2, a2_q=a2_q, a2_s=a2_s,

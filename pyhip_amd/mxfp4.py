@@ -97,3 +97,47 @@ def prepare_expert_weights(w, shuffle=True):
         q = shuffle_weight(q)
         q.is_shuffled = True
     return q, e8m0_shuffle(s.reshape(E * N, K // BLOCK))
+
+
+def pad_to(n, multiple=512):
+    return (n + multiple - 1) // multiple * multiple
+
+
+def pad_layer_weights(w1q, w1s, w2q, w2s, bias1=None, bias2=None, multiple=512):
+    """Zero-pad quantised (not yet shuffled) expert weights so that ``hidden`` and ``inter`` become
+    multiples of ``multiple``, the way aiter pads gpt-oss weights (hidden 2880 -> 3072): the caller then
+    passes ``hidden_pad`` / ``intermediate_pad`` to ``fused_moe`` (reference argument meaning:
+    tests/contrib/moe/test_fused_moe.py:92-105 -- the trailing rows/columns of the padded weights are zero).
+
+    w1q uint8 [E, 2I, H/2] (gate rows then up rows), w1s uint8 [E, 2I, H/32], w2q [E, H, I/2], w2s [E, H, I/32].
+    Returns (w1q, w1s, w2q, w2s, bias1, bias2, hidden_pad, intermediate_pad) at the padded sizes; gate rows stay
+    at [0, I), up rows move to [I_padded, I_padded + I).  A zero byte is the e2m1 pair (0, 0) and a zero
+    scale byte multiplies it by 2^-127, so padded rows and columns contribute exactly nothing."""
+    E, N1, Hb = w1q.shape
+    H, I = Hb * 2, N1 // 2
+    Hp, Ip = pad_to(H, multiple), pad_to(I, multiple)
+    if (Hp, Ip) == (H, I):
+        return w1q, w1s, w2q, w2s, bias1, bias2, 0, 0
+
+    def grow(t, rows_from, rows_to, cols):
+        out = torch.zeros(t.shape[0], rows_to, cols, dtype=t.dtype, device=t.device)
+        out[:, :rows_from, : t.shape[2]] = t
+        return out
+
+    def grow_gate_up(t, cols):
+        out = torch.zeros(t.shape[0], 2 * Ip, cols, dtype=t.dtype, device=t.device)
+        out[:, :I, : t.shape[2]] = t[:, :I]
+        out[:, Ip:Ip + I, : t.shape[2]] = t[:, I:]
+        return out
+
+    w1q_p, w1s_p = grow_gate_up(w1q, Hp // 2), grow_gate_up(w1s, Hp // BLOCK)
+    w2q_p, w2s_p = grow(w2q, H, Hp, Ip // 2), grow(w2s, H, Hp, Ip // BLOCK)
+    if bias1 is not None:
+        b = torch.zeros(E, 2 * Ip, dtype=bias1.dtype, device=bias1.device)
+        b[:, :I], b[:, Ip:Ip + I] = bias1[:, :I], bias1[:, I:]
+        bias1 = b
+    if bias2 is not None:
+        b = torch.zeros(E, Hp, dtype=bias2.dtype, device=bias2.device)
+        b[:, :H] = bias2
+        bias2 = b
+    return w1q_p, w1s_p, w2q_p, w2s_p, bias1, bias2, Hp - H, Ip - I

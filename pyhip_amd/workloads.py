@@ -59,29 +59,32 @@ def make_weights(shape, device="cuda", seed=0, experts_per_chunk=8):
     Weights are drawn and quantised chunk by chunk; fp32 copies of all experts never coexist."""
     cfg = SHAPES[shape] if isinstance(shape, str) else shape
     E, H, I = cfg["E"], cfg["H"], cfg["I"]
+    Hp, Ip = mxfp4.pad_to(H), mxfp4.pad_to(I)      # the GEMMs tile K by 512: gpt-oss 2880 -> 3072
     g = torch.Generator(device=device).manual_seed(seed)
-    w1 = torch.empty(E, 2 * I, H // 2, dtype=torch.uint8, device=device)
-    w2 = torch.empty(E, H, I // 2, dtype=torch.uint8, device=device)
-    s1 = torch.empty(E * 2 * I, H // 32, dtype=torch.uint8, device=device)
-    s2 = torch.empty(E * H, I // 32, dtype=torch.uint8, device=device)
+    w1 = torch.empty(E, 2 * Ip, Hp // 2, dtype=torch.uint8, device=device)
+    w2 = torch.empty(E, Hp, Ip // 2, dtype=torch.uint8, device=device)
+    s1 = torch.empty(E * 2 * Ip, Hp // 32, dtype=torch.uint8, device=device)
+    s2 = torch.empty(E * Hp, Ip // 32, dtype=torch.uint8, device=device)
     for e0 in range(0, E, experts_per_chunk):
         e1 = min(E, e0 + experts_per_chunk)
-        x = torch.randn(e1 - e0, 2 * I, H, generator=g, device=device) * 0.02
-        q, s = mxfp4.quantize_mxfp4(x)
-        w1[e0:e1] = mxfp4.shuffle_weight(q)
-        s1[e0 * 2 * I:e1 * 2 * I] = s.reshape(-1, H // 32)
-        x = torch.randn(e1 - e0, H, I, generator=g, device=device) * 0.02
-        q, s = mxfp4.quantize_mxfp4(x)
-        w2[e0:e1] = mxfp4.shuffle_weight(q)
-        s2[e0 * H:e1 * H] = s.reshape(-1, I // 32)
-        del x, q, s
+        q1, sc1 = mxfp4.quantize_mxfp4(torch.randn(e1 - e0, 2 * I, H, generator=g, device=device) * 0.02)
+        q2, sc2 = mxfp4.quantize_mxfp4(torch.randn(e1 - e0, H, I, generator=g, device=device) * 0.02)
+        q1, sc1, q2, sc2 = mxfp4.pad_layer_weights(q1, sc1, q2, sc2)[:4]
+        w1[e0:e1] = mxfp4.shuffle_weight(q1)
+        s1[e0 * 2 * Ip:e1 * 2 * Ip] = sc1.reshape(-1, Hp // 32)
+        w2[e0:e1] = mxfp4.shuffle_weight(q2)
+        s2[e0 * Hp:e1 * Hp] = sc2.reshape(-1, Ip // 32)
+        del q1, sc1, q2, sc2
     w1.is_shuffled = True
     w2.is_shuffled = True
     out = dict(w1=w1, w2=w2, w1_scale=mxfp4.e8m0_shuffle(s1), w2_scale=mxfp4.e8m0_shuffle(s2),
-               w1_scale_plain=s1, w2_scale_plain=s2)
+               w1_scale_plain=s1, w2_scale_plain=s2, hidden_pad=Hp - H, intermediate_pad=Ip - I)
     if cfg.get("bias"):
-        out["bias1"] = (torch.randn(E, 2 * I, generator=g, device=device) * 0.01).to(torch.bfloat16)
-        out["bias2"] = (torch.randn(E, H, generator=g, device=device) * 0.01).to(torch.bfloat16)
+        b1 = (torch.randn(E, 2 * I, generator=g, device=device) * 0.01).to(torch.bfloat16)
+        b2 = (torch.randn(E, H, generator=g, device=device) * 0.01).to(torch.bfloat16)
+        out["bias1"] = torch.zeros(E, 2 * Ip, dtype=torch.bfloat16, device=device)
+        out["bias1"][:, :I], out["bias1"][:, Ip:Ip + I] = b1[:, :I], b1[:, I:]
+        out["bias2"] = torch.nn.functional.pad(b2, (0, Hp - H))
     return out
 
 

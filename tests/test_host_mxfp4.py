@@ -41,3 +41,34 @@ def test_prepare_expert_weights():
     oq, os_ = om.quantize_mxfp4(w.numpy())
     assert (q.numpy() == ol.shuffle_weight(oq)).all()
     assert (s.numpy() == ol.e8m0_shuffle(os_.reshape(256, 4))).all()
+
+
+def test_pad_layer_weights_is_exact():
+    """zero-padding quantised weights changes nothing: dequantised padded weights are the originals
+    surrounded by zeros, gate/up halves land where the padded layout expects them"""
+    from oracle import mxfp4 as om
+    rng = np.random.default_rng(5)
+    E, H, I = 3, 96, 160
+    w1 = (rng.standard_normal((E, 2 * I, H)) * 0.02).astype(np.float32)
+    w2 = (rng.standard_normal((E, H, I)) * 0.02).astype(np.float32)
+    w1q, w1s = om.quantize_mxfp4(w1)
+    w2q, w2s = om.quantize_mxfp4(w2)
+    b1 = torch.arange(E * 2 * I, dtype=torch.float32).reshape(E, 2 * I).to(torch.bfloat16)
+    b2 = torch.arange(E * H, dtype=torch.float32).reshape(E, H).to(torch.bfloat16)
+    t = torch.from_numpy
+    pm = mxfp4
+    p1q, p1s, p2q, p2s, pb1, pb2, hp, ip = pm.pad_layer_weights(t(w1q), t(w1s), t(w2q), t(w2s), b1, b2, multiple=128)
+    Hp, Ip = 128, 256
+    assert (hp, ip) == (Hp - H, Ip - I)
+    d1 = om.dequantize_mxfp4(p1q.numpy(), p1s.numpy())
+    d2 = om.dequantize_mxfp4(p2q.numpy(), p2s.numpy())
+    o1, o2 = om.dequantize_mxfp4(w1q, w1s), om.dequantize_mxfp4(w2q, w2s)
+    assert d1.shape == (E, 2 * Ip, Hp) and d2.shape == (E, Hp, Ip)
+    assert (d1[:, :I, :H] == o1[:, :I]).all() and (d1[:, Ip:Ip + I, :H] == o1[:, I:]).all()
+    assert d1.sum() == o1.sum() and np.abs(d1).sum() == np.abs(o1).sum()          # everything else is zero
+    assert (d2[:, :H, :I] == o2).all() and np.abs(d2).sum() == np.abs(o2).sum()
+    assert (pb1[:, :I] == b1[:, :I]).all() and (pb1[:, Ip:Ip + I] == b1[:, I:]).all() and pb1.float().abs().sum() == b1.float().abs().sum()
+    assert (pb2[:, :H] == b2).all() and (pb2[:, H:] == 0).all()
+    # already aligned: returned unchanged
+    same = pm.pad_layer_weights(t(w1q), t(w1s), t(w2q), t(w2s), multiple=32)
+    assert same[0].data_ptr() == t(w1q).data_ptr() and same[6:] == (0, 0)
