@@ -66,11 +66,15 @@ __device__ __forceinline__ void wave_hist(const SortArgs& a, u32* h, int beg, in
 }
 
 // writes the pairs [beg, end) to their final positions; base[e] (LDS, private to this wave) is the
-// position of the wave's first pair of expert e and is advanced as groups are consumed
+// position of the wave's first pair of expert e and is advanced as groups are consumed.  Within a
+// group of 64 pairs every lane finds the lanes that hold the same expert from one ballot per bit of
+// the expert id (a constant number of steps, however many distinct experts the group holds); its rank
+// among them gives the position, and the lowest such lane advances base[e].
 __device__ __forceinline__ void wave_scatter(const SortArgs& a, u32* base, int beg, int end)
 {
     const int lane  = lane_id();
     const u64 lt    = (1ull << lane) - 1ull;
+    const int nbits = 32 - __builtin_clz((unsigned)(a.E > 1 ? a.E - 1 : 1));
     for(int g = beg; g < end; g += WAVE)
     {
         int i     = g + lane;
@@ -81,25 +85,24 @@ __device__ __forceinline__ void wave_scatter(const SortArgs& a, u32* base, int b
             e = a.topk_ids[i];
             w = a.topk_w[i];
         }
-        bool keep = e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
-        u64 todo  = __ballot(keep);
-        while(todo)
+        const bool keep = e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
+        u64 m           = __ballot(keep);
+        for(int b = 0; b < nbits; b++)
         {
-            int leader = __ffsll((long long)todo) - 1;
-            int el     = __shfl(e, leader);
-            u64 m      = __ballot(keep && e == el);
-            if(keep && e == el)
-            {
-                u32 pos          = base[el] + (u32)__popcll(m & lt);
-                u32 tok          = (u32)(i / a.k);
-                u32 slot         = (u32)(i - (int)tok * a.k);
-                a.sorted_ids[pos] = (slot << 24) | tok;
-                a.sorted_w[pos]   = w;
-            }
-            if(lane == leader)
-                base[el] += (u32)__popcll(m);
-            todo &= ~m;
+            const bool bit = (e >> b) & 1;
+            const u64 bal  = __ballot(keep && bit);
+            m &= bit ? bal : ~bal;
         }
+        if(keep)
+        {
+            const u32 pos     = base[e] + (u32)__popcll(m & lt);
+            const u32 tok     = (u32)(i / a.k);
+            const u32 slot    = (u32)(i - (int)tok * a.k);
+            a.sorted_ids[pos] = (slot << 24) | tok;
+            a.sorted_w[pos]   = w;
+        }
+        if(keep && (m & lt) == 0)       // lowest lane of its expert; every lane above has read base[e] already
+            base[e] += (u32)__popcll(m);
     }
 }
 
@@ -316,11 +319,19 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
     {
         u32 run = 0;
-        for(int g = 0; g < a.G; g++)
+        for(int g0 = 0; g0 < a.G; g0 += 16)      // 16 independent loads in flight, then their prefix
         {
-            u32 c                    = a.ws[(size_t)g * a.E + e];
-            a.ws[(size_t)g * a.E + e] = run;
-            run += c;
+            u32 c[16];
+#pragma unroll
+            for(int j = 0; j < 16; j++)
+                c[j] = g0 + j < a.G ? __builtin_nontemporal_load(&a.ws[(size_t)(g0 + j) * a.E + e]) : 0u;
+#pragma unroll
+            for(int j = 0; j < 16; j++)
+                if(g0 + j < a.G)
+                {
+                    a.ws[(size_t)(g0 + j) * a.E + e] = run;
+                    run += c[j];
+                }
         }
         tot[e] = run;
     }
@@ -380,9 +391,9 @@ extern "C" __global__ void moe_zero_kernel(uint4* p, size_t n16, unsigned char* 
 
 static int sort_groups(int64_t pairs)
 {
-    // workgroups of the large path: 256 pairs per wave-chunk minimum, at most 128 workgroups
-    int64_t g = (pairs + SORT_THREADS * 4 - 1) / (SORT_THREADS * 4);
-    return (int)(g < 1 ? 1 : (g > 128 ? 128 : g));
+    // workgroups of the large path: at least 1024 pairs each (4 groups of 64 per wave), at most 256 workgroups
+    int64_t g = (pairs + 1023) / 1024;
+    return (int)(g < 1 ? 1 : (g > 256 ? 256 : g));
 }
 
 extern "C" int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size)
