@@ -77,15 +77,20 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
  *                src/misc.py:116-130 (pre_shuffle(x, 16))
  *   w1_scale     e8m0, shuffled as tests/contrib/moe/test_fused_moe.py:222-236 over [experts*2*inter, hidden/32]
  *   bias1        bf16 [experts, 2*inter] or NULL
- *   a2           bf16 [n_blk*block_m, inter], row = sorted position (padding rows are zero)
+ *   a2           bf16 [n_blk*block_m, inter], row = sorted position (padding rows are zero); may be NULL
+ *   a2_q/a2_scale  (both or neither; may be NULL) the MXFP4 quantisation of a2 in the layout of
+ *                pyhip_moe_act_quant_mxfp4, written by the same kernel: bit-identical to quantising a2
+ *                afterwards, and it replaces the second aiter.get_hip_quant + moe_mxfp4_sort call of
+ *                tests/contrib/moe/test_moe.py:732-744.  Needs inter % 512 == 0.  At least one of a2 and
+ *                a2_q must be given.
  * block_m must equal the block_size the sort ran with and `experts` the expert count it ran with;
  * block_m is 16, 32, 64 or 128; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
  * workgroup per tile and worst-case block is launched, as the reference does). */
 int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
-                          const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, int tokens,
-                          int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
-                          pyhip_stream_t stream);
+                          const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q,
+                          uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                          int64_t n_blk, pyhip_stream_t stream);
 
 /* Stage 2: down grouped GEMM, times the routing weight.  Replaces moe_gemm_mxfp4(gate_up=False),
  * src/contrib/moe_gemm_mxfp4.py:1291-1333 (launch: tests/contrib/moe/test_moe.py:751-763).

@@ -56,6 +56,40 @@ __device__ __forceinline__ float silu_f32(float x)
     return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// ---- MXFP4 quantisation of bf16 values (shared by the quantisation kernel and the stage-1 GEMM epilogue)
+// running maximum of the magnitudes (15-bit patterns) of the two bf16 halves of w
+__device__ __forceinline__ u32 amax15(u32 acc, u32 w)
+{
+    u32 lo = w & 0x7FFFu, hi = (w >> 16) & 0x7FFFu;
+    acc    = acc > lo ? acc : lo;
+    return acc > hi ? acc : hi;
+}
+
+// eight bf16 (one uint4) times a power of two -> eight e2m1 codes in one dword
+__device__ __forceinline__ u32 cvt8(uint4 v, float mul)
+{
+    u32 r = 0;
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.x & 0xFFFFu) * mul,
+                                                 bf16_bits_to_f32(v.x >> 16) * mul, 1.0f, 0);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.y & 0xFFFFu) * mul,
+                                                 bf16_bits_to_f32(v.y >> 16) * mul, 1.0f, 1);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.z & 0xFFFFu) * mul,
+                                                 bf16_bits_to_f32(v.z >> 16) * mul, 1.0f, 2);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.w & 0xFFFFu) * mul,
+                                                 bf16_bits_to_f32(v.w >> 16) * mul, 1.0f, 3);
+    return r;
+}
+
+// e8m0 scale byte of a block whose largest bf16 magnitude pattern is am: 2^(floor(log2 amax) - 2), byte 0 for amax < 2^-124
+__device__ __forceinline__ u32 mx_scale_byte(u32 am)
+{
+    int ex = (int)(am >> 7);                             // biased exponent of amax (bf16: 8 exponent bits)
+    u32 e8 = (u32)(ex > 2 ? ex - 2 : 0);
+    return e8 > 254u ? 254u : e8;
+}
+// x / 2^(e8-127) = x * 2^(127-e8): exponent field 254-e8 is in [1, 254], always a normal float
+__device__ __forceinline__ float mx_inv_scale(u32 e8) { return __builtin_bit_cast(float, (254u - e8) << 23); }
+
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
 
 // compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{})

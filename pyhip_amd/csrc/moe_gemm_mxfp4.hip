@@ -37,7 +37,10 @@ struct GemmArgs
     const u32* sorted_e;       // [n_blk]
     const u32* num_valid;      // [2]
     const u32* sched;          // tile schedule written by the sort (moe_sort.hip: write_schedule) or null
-    void* out;                 // stage 1: bf16 [n_blk*BM, N/2]; stage 2: bf16 [T, topk, N]
+    void* out;                 // stage 1: bf16 [n_blk*BM, N/2] (may be null); stage 2: bf16 [T, topk, N]
+    uint8_t* out_q;            // stage 1: MXFP4 of the output, e2m1 pairs [n_blk*BM, N/4], or null
+    uint8_t* out_s;            //          and its scales [n_blk*BM, OSK] in the activation-scale layout
+    int OSK;
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
 #ifdef PYHIP_GEMM_DEBUG
     int dbg;
@@ -413,7 +416,27 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                 v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
                 v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
                 // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
-                *(uint4*)(out + (size_t)p * I + ch_out) = make_uint4(t0.x, t1.x, t0.y, t1.y);
+                const uint4 o = make_uint4(t0.x, t1.x, t0.y, t1.y);
+                if(out)
+                    *(uint4*)(out + (size_t)p * I + ch_out) = o;
+                if(g.out_q)
+                {
+                    // the wave's 32 channels of a row are exactly one MX block (8 channels in each of the four
+                    // lane rows): block maximum across the lane rows, then the same arithmetic as the stand-alone
+                    // quantiser (moe_quant.hip) on the bf16-rounded values, so both paths agree bit for bit
+                    u32 am = amax15(amax15(amax15(amax15(0u, o.x), o.y), o.z), o.w);
+                    v2u s16 = __builtin_amdgcn_permlane16_swap(am, am, false, false);
+                    am      = s16.x > s16.y ? s16.x : s16.y;
+                    v2u s32 = __builtin_amdgcn_permlane32_swap(am, am, false, false);
+                    am      = s32.x > s32.y ? s32.x : s32.y;
+                    const u32 e8 = mx_scale_byte(am);
+                    *(u32*)(g.out_q + (size_t)p * (I / 2) + ch_out / 2) = cvt8(o, mx_inv_scale(e8));
+                    if(kb == 0)
+                    {
+                        const int blk = t.nt * 4 + wave, jb = blk & 15;      // scale byte: see moe_quant.hip
+                        g.out_s[(size_t)p * g.OSK + (blk & ~15) + (jb & 3) * 4 + (jb >> 2)] = (uint8_t)e8;
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
             }
         }
@@ -695,11 +718,16 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1,
                                      const uint8_t* w1_scale, const void* bias1_bf16, const uint32_t* sorted_ids,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
-                                     const uint32_t* schedule, void* a2_bf16, int tokens, int topk, int experts,
-                                     int hidden, int inter, int block_m, int64_t n_blk, hipStream_t stream)
+                                     const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q, uint8_t* a2_scale,
+                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                     int64_t n_blk, hipStream_t stream)
 {
+    PYHIP_REQUIRE(a2_bf16 || a2_q, "moe_gemm1: no output buffer");
+    PYHIP_REQUIRE((a2_q == nullptr) == (a2_scale == nullptr), "moe_gemm1: a2_q and a2_scale go together");
+    PYHIP_REQUIRE(!a2_q || inter % 512 == 0, "moe_gemm1: quantised output needs inter=%d to be a multiple of 512", inter);
+    PYHIP_REQUIRE(((uintptr_t)a2_q % 4) == 0 && ((uintptr_t)a2_bf16 % 16) == 0, "moe_gemm1: unaligned output");
     int rc = check_common("moe_gemm1", a_q, a_scale, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
-                          a2_bf16, hidden, block_m, n_blk, tokens);
+                          a2_bf16 ? a2_bf16 : (void*)a2_q, hidden, block_m, n_blk, tokens);
     if(rc)
         return rc;
     PYHIP_REQUIRE(inter > 0 && inter % 128 == 0, "moe_gemm1: inter=%d must be a multiple of 128", inter);
@@ -709,7 +737,8 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
     GemmArgs g;
     g.a_q = a_q; g.a_s = a_scale; g.w = w1; g.w_s = w1_scale; g.bias = (const uint16_t*)bias1_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
-    g.out = a2_bf16; g.sched = schedule; g.E = experts;
+    g.out = a2_bf16; g.out_q = a2_q; g.out_s = a2_scale; g.OSK = (inter + 511) / 512 * 16;
+    g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
     g.SK = (hidden + 511) / 512 * 16;
     g.SC = (hidden / 32 + 7) / 8 * 8;
@@ -736,7 +765,8 @@ extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scal
     GemmArgs g;
     g.a_q = a2_q; g.a_s = a2_scale; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
-    g.num_valid = num_valid_ids; g.out = out3_bf16; g.sched = schedule; g.E = experts;
+    g.num_valid = num_valid_ids; g.out = out3_bf16; g.out_q = nullptr; g.out_s = nullptr; g.OSK = 0;
+    g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = inter; g.N = hidden;
     g.SK = (inter + 511) / 512 * 16;
     g.SC = (inter / 32 + 7) / 8 * 8;

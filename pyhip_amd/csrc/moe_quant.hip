@@ -14,28 +14,6 @@
 
 #define QUANT_THREADS 256
 
-__device__ __forceinline__ u32 amax15(u32 acc, u32 w)
-{
-    u32 lo = w & 0x7FFFu, hi = (w >> 16) & 0x7FFFu;
-    acc    = acc > lo ? acc : lo;
-    return acc > hi ? acc : hi;
-}
-
-// eight bf16 (one uint4) times a power of two -> eight e2m1 codes in one dword
-__device__ __forceinline__ u32 cvt8(uint4 v, float mul)
-{
-    u32 r = 0;
-    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.x & 0xFFFFu) * mul,
-                                                 bf16_bits_to_f32(v.x >> 16) * mul, 1.0f, 0);
-    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.y & 0xFFFFu) * mul,
-                                                 bf16_bits_to_f32(v.y >> 16) * mul, 1.0f, 1);
-    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.z & 0xFFFFu) * mul,
-                                                 bf16_bits_to_f32(v.z >> 16) * mul, 1.0f, 2);
-    r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, bf16_bits_to_f32(v.w & 0xFFFFu) * mul,
-                                                 bf16_bits_to_f32(v.w >> 16) * mul, 1.0f, 3);
-    return r;
-}
-
 // one thread per 32-element block; 16 consecutive threads own one 16-byte scale group
 extern "C" __global__ void __launch_bounds__(QUANT_THREADS)
     moe_act_quant_mxfp4_kernel(const uint16_t* __restrict__ x, long long ldx, uint8_t* __restrict__ q,
@@ -62,11 +40,8 @@ extern "C" __global__ void __launch_bounds__(QUANT_THREADS)
         am = amax15(am, v1.x); am = amax15(am, v1.y); am = amax15(am, v1.z); am = amax15(am, v1.w);
         am = amax15(am, v2.x); am = amax15(am, v2.y); am = amax15(am, v2.z); am = amax15(am, v2.w);
         am = amax15(am, v3.x); am = amax15(am, v3.y); am = amax15(am, v3.z); am = amax15(am, v3.w);
-        int ex = (int)(am >> 7);                         // biased exponent of amax (bf16: 8 exponent bits)
-        e8     = (u32)(ex > 2 ? ex - 2 : 0);
-        e8     = e8 > 254u ? 254u : e8;
-        // x / 2^(e8-127) = x * 2^(127-e8): exponent field 254-e8 is in [1, 254], always a normal float
-        float mul = __builtin_bit_cast(float, (254u - e8) << 23);
+        e8        = mx_scale_byte(am);
+        float mul = mx_inv_scale(e8);
         uint4 o;
         o.x = cvt8(v0, mul);
         o.y = cvt8(v1, mul);

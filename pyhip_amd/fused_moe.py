@@ -136,19 +136,20 @@ def fused_moe(
         assert tuple(bias2.shape) == (E, H)
 
     a1_q, a1_s = act_quant_mxfp4(hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous())
-    a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
+    # the stage-1 kernel writes its result already quantised for stage 2; the bf16 copy is only produced on request
+    a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev) if return_parts else None
+    a2_q = torch.empty(n_blk * bm, I // 2, dtype=torch.uint8, device=dev)
+    a2_s = torch.empty(n_blk * bm, lib.pyhip_moe_act_scale_stride(I), dtype=torch.uint8, device=dev)
     ev = _mark("quant1", ev)
     rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                    _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
-                                   _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), T, k, global_E, H, I, bm,
-                                   n_blk, stream)
+                                   _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
+                                   _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
-    a2_q, a2_s = act_quant_mxfp4(a2, rows_limit=num_valid)
     out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
     if expert_mask is not None or num_local_tokens is not None:
         out3.zero_()          # slots routed to experts this rank does not hold contribute nothing
-    ev = _mark("quant2", ev)
     rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
                                    _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
                                    _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),

@@ -144,6 +144,14 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
     assert (parts["a1_q"].cpu().numpy() == oq).all()
     assert (cases.untranspose_act_scales(parts["a1_s"].cpu().numpy(), L.H) == os_).all()
 
+    # the quantised copy of the stage-1 result written by the GEMM epilogue is what the stand-alone quantiser
+    # makes of the bf16 copy, bit for bit
+    nv = int(parts["num_valid_ids"][0])
+    q2, s2 = act_quant_mxfp4(parts["a2"][:nv].contiguous())
+    assert torch.equal(parts["a2_q"][:nv], q2) and torch.equal(parts["a2_s"][:nv], s2)
+    oq2, os2 = om.quantize_mxfp4(_f(parts["a2"][:nv]))
+    assert (q2.cpu().numpy() == oq2).all() and (cases.untranspose_act_scales(s2.cpu().numpy(), L.I) == os2).all()
+
     # stage-wise, each stage fed the kernel's own previous output
     w1e, w2e, ref_a2 = _stage_checks(L, parts, parts["block_m"])
     assert w1e <= TOL_MAX, f"stage 1 (max|err| - ulp)/rms = {w1e}"
