@@ -6,6 +6,7 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
 
   value     TFLOP/s of the whole layer at --tokens (default 8192), FLOPs = 6*T*k*I*H
   decode    the same layer at --decode-tokens (default 16): ms, HBM GB/s on algorithmic bytes
+  decode_w4a16  the same with bf16 activations (method="w4a16")
   roofline  the dominant kernel (stage-1 gate_up GEMM) of the primary workload, timed with events
             recorded around it inside the timed steps
   cpu_baseline  the CPU oracle (oracle/moe.py) on a bounded sample of the same workload
@@ -38,13 +39,14 @@ def parse():
     return ap.parse_args()
 
 
-def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m):
+def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, method="auto"):
     from pyhip_amd import workloads
     hidden, topk_w, topk_ids = workloads.make_inputs(shape, tokens)
     if W["hidden_pad"]:      # padded shapes (gpt-oss): activations at the padded width, as the reference passes them
         hidden = torch.nn.functional.pad(hidden, (0, W["hidden_pad"]))
     kw = dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
-              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"])
+              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"],
+              method=method)
     for _ in range(warmup):
         out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, **kw)
     torch.cuda.synchronize()
@@ -125,6 +127,7 @@ def main():
     torch.cuda.synchronize()
     main_res = run_config(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m)
     dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
+    dec16 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), 0, "w4a16")
 
     if a.calibrate_copy:
         src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
@@ -165,6 +168,10 @@ def main():
                                 "frac": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                                 "traffic": None, "avg_launch_ms": round(dg1_ms, 4)}},
     }
+    out["decode_w4a16"] = {"tokens": a.decode_tokens, "ms_per_step": round(dec16["ms"], 4),
+                           "hbm_gbps": round(dw["bytes"] / (dec16["ms"] * 1e-3) / 1e9, 1),
+                           "frac_of_hbm_peak": round(dw["bytes"] / (dec16["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                           "stage_ms": {k: round(v, 4) for k, v in dec16["stage_ms"].items()}}
     if a.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds)
     print(json.dumps(out))

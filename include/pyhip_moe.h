@@ -106,6 +106,23 @@ int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const ui
                           int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The same two GEMMs with bf16 activations ("w4a16"): weights are expanded from MXFP4 to bf16 in registers
+ * and multiplied with the bf16 MFMA; nothing is quantised at run time.  Replaces moe_2stage_splitk with fp4
+ * weights, src/contrib/moe.py:362-787 (gate_up: with_silu=True; down: :471-500,703-787; launches:
+ * tests/contrib/moe/test_moe.py:347-374), the variant the reference uses when few tokens are routed.
+ * Buffers as above, except hidden / a2 are bf16 ([tokens, hidden] in token order; [n_blk*block_m, inter] in
+ * sorted-row order) and the down GEMM writes out3[tokens, topk, hidden] for pyhip_moe_topk_reduce instead of
+ * adding into the layer output with atomics.  block_m is 16, 32 or 64; hidden % 512 == 0, inter % 512 == 0. */
+int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale, const void* bias1_bf16,
+                          const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
+                          void* a2_bf16, int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                          int64_t n_blk, pyhip_stream_t stream);
+int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale, const void* bias2_bf16,
+                          const uint32_t* sorted_ids, const float* sorted_weights, const uint32_t* sorted_expert_ids,
+                          const uint32_t* num_valid_ids, void* out3_bf16, int tokens, int topk, int experts,
+                          int hidden, int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.
  * Replaces moe_gemm_final_reduce_bf16, src/contrib/moe_gemm_mxfp4.py:199-282
  * (launch: tests/contrib/moe/test_moe.py:764-771).  out is bf16 or (out_is_f32 != 0) fp32.

@@ -535,7 +535,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                 setup_null();
         }
 #ifdef PYHIP_GEMM_DEBUG
-        if(g.dbg & 3) setup_null();
+        if(g.dbg & 1) { wrs[0] = wrs[1] = make_rsrc(g.w, 0); wsrs[0] = wsrs[1] = make_rsrc(g.w_s, 0); }
+        if(g.dbg & 2) { ars = make_rsrc(g.a_q, 0); asrs = make_rsrc(g.a_s, 0); }
 #endif
         const bool meta_on = ks == 0 && nxt.valid;
         const v4i rid = make_rsrc(g.sorted_ids + (size_t)nxt.m_blk * BM, BM * 4);

@@ -1,0 +1,271 @@
+// Grouped GEMMs of the fused-MoE layer with bf16 activations and MXFP4 weights ("w4a16"): the weights are
+// expanded to bf16 in registers (e2m1 value times its e8m0 block scale is exact in bf16) and multiplied with
+// the bf16 MFMA.  This is the variant the reference runs when few tokens are routed
+// (src/contrib/moe.py:362-787, moe_2stage_splitk with fp4 weights, driven by
+// tests/contrib/moe/test_moe.py:347-374); at such sizes the layer only streams weights, so the kernel is kept
+// simple: one workgroup per (row block, weight tile), the K loop software-pipelined one K-step ahead, no LDS.
+//
+// Operand mapping.  A pre-shuffled 1 KB weight block (src/misc.py:116-130) gives lane (row = l % 16,
+// kb = l / 16) the 32 consecutive K-elements kb*32 .. kb*32+31 of its row.  The bf16 MFMA 16x16x32 wants 8
+// K-elements per lane, so one block feeds four MFMAs; in MFMA i the lane contributes elements
+// kb*32 + i*8 .. +7, and the token side loads the same elements of its activation row (16 contiguous bytes).
+// Any fixed pairing of K-elements is a valid contraction order.  Weights are src A and tokens src B, so a lane
+// ends with 4 consecutive output channels of token l % 16, as in the MXFP4-activation kernel.
+#include "common.h"
+
+#define W4A16_THREADS 256
+
+struct W4A16Args
+{
+    const uint16_t* a;         // activations bf16: stage 1 [T, K] (token order); stage 2 [n_blk*BM, K] (sorted order)
+    const uint8_t* w;          // weights, pre-shuffled    [E, N, K/2]
+    const uint8_t* w_s;        // weight scales, shuffled  [E*N (padded to 256), SC]
+    const uint16_t* bias;      // bf16 [E, N] or null
+    const u32* sorted_ids;     // [n_blk * BM]
+    const float* sorted_w;     // [n_blk * BM] (stage 2)
+    const u32* sorted_e;       // [n_blk]
+    const u32* num_valid;      // [2]
+    uint16_t* out;             // stage 1: bf16 [n_blk*BM, N/2]; stage 2: bf16 [T, topk, N]
+    int T, topk, K, N, SC, n_tiles;
+};
+
+// 32 e2m1 values (4 dwords) times 2^(scale byte - 127) -> four MFMA operands of 8 bf16
+__device__ __forceinline__ void expand_fp4(const v4i& w, u32 scale_byte, v8bf (&o)[4])
+{
+    const float sc = __builtin_bit_cast(float, scale_byte << 23);
+#pragma unroll
+    for(int i = 0; i < 4; i++)
+    {
+        const u32 d = (u32)w[i];
+        v2bf p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, sc, 0);
+        v2bf p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, sc, 1);
+        v2bf p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, sc, 2);
+        v2bf p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, sc, 3);
+        o[i] = (v8bf){p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+    }
+}
+
+// STAGE 1 = gate_up (+ SiLU(gate) * up), 2 = down (* routing weight).  MT = row groups of 16 per tile.
+template <int STAGE, int MT>
+__global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
+{
+    constexpr int BM = MT * 16;
+    const int tid = threadIdx.x, lane = tid % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int r = lane & 15, kb = lane >> 4;
+    const int m_blk = blockIdx.x / g.n_tiles, nt = blockIdx.x - m_blk * g.n_tiles;
+    if((u32)(m_blk * BM) >= g.num_valid[0])
+        return;
+    const int e  = (int)g.sorted_e[m_blk];
+    const int Kb = g.K / 2, I = g.N / 2;
+
+    // weight row groups of this wave: j = 0..3 (stage 1: j>>1 selects gate / up)
+    const uint8_t* wp[4];
+    const uint8_t* sp[4];      // scale tile row (32 weight rows) of row group j
+    int sbyte_row[4];          // which 16-row half of the 32-row scale tile
+    const size_t sc_tile = (size_t)(g.SC / 8) * 256;
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+    {
+        const size_t row = STAGE == 1 ? (size_t)e * g.N + (j >> 1) * I + nt * 128 + wave * 32 + (j & 1) * 16
+                                      : (size_t)e * g.N + nt * 256 + wave * 64 + j * 16;
+        wp[j]        = g.w + row * Kb + lane * 16;
+        sp[j]        = g.w_s + (row / 32) * sc_tile + lane * 4;
+        sbyte_row[j] = (int)((row / 16) & 1);
+    }
+    // activation rows of this lane, one per row group
+    const uint16_t* ap[MT];
+    bool ok[MT];
+    u32 ids[MT];
+#pragma unroll
+    for(int mt = 0; mt < MT; mt++)
+    {
+        const int p  = m_blk * BM + mt * 16 + r;
+        ids[mt]      = g.sorted_ids[p];
+        const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
+        ok[mt]       = slot < g.topk && tok < g.T;
+        const size_t row = STAGE == 1 ? (size_t)(ok[mt] ? tok : 0) : (size_t)p;
+        ap[mt]       = g.a + row * g.K + kb * 32;
+    }
+
+    v4f acc[4][MT];
+#pragma unroll
+    for(int j = 0; j < 4; j++)
+#pragma unroll
+        for(int mt = 0; mt < MT; mt++)
+            acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    const int KT = g.K / 128;
+    v4i wf[2][4];
+    v4i af[2][MT][4];
+    u32 wsc[4];                // scale dwords of the current 256-K column tile (two K-steps)
+    auto load_step = [&](int buf, int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            wf[buf][j] = __builtin_nontemporal_load((const v4i*)(wp[j] + (size_t)kt * 1024));
+#pragma unroll
+        for(int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+                af[buf][mt][i] = *(const v4i*)(ap[mt] + kt * 128 + i * 8);
+    };
+    load_step(0, 0);
+    for(int kt = 0; kt < KT; kt++)
+    {
+        const int cur = kt & 1;
+        if((kt & 1) == 0)
+        {
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+                wsc[j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
+        }
+        if(kt + 1 < KT)
+        {
+            if(cur == 0)
+                load_step(1, kt + 1);
+            else
+                load_step(0, kt + 1);
+        }
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+        {
+            // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
+            const u32 sb = (wsc[j] >> (8 * ((kt & 1) * 2 + sbyte_row[j]))) & 0xFFu;
+            v8bf wq[4];
+            if(cur == 0)
+                expand_fp4(wf[0][j], sb, wq);
+            else
+                expand_fp4(wf[1][j], sb, wq);
+#pragma unroll
+            for(int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for(int i = 0; i < 4; i++)
+                {
+                    const v4i av = cur == 0 ? af[0][mt][i] : af[1][mt][i];
+                    acc[j][mt]   = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wq[i], __builtin_bit_cast(v8bf, av),
+                                                                         acc[j][mt], 0, 0, 0);
+                }
+        }
+    }
+
+    // ---- epilogue: lane (r, kb) holds channels kb*4 .. kb*4+3 of row group j for token row r
+    if(g.bias)
+    {
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int i = 0; i < 4; i++)
+            {
+                const int ch = STAGE == 1 ? (j >> 1) * I + nt * 128 + wave * 32 + (j & 1) * 16 + kb * 4 + i
+                                          : nt * 256 + wave * 64 + j * 16 + kb * 4 + i;
+                const float b = bf16_bits_to_f32(g.bias[(size_t)e * g.N + ch]);
+#pragma unroll
+                for(int mt = 0; mt < MT; mt++)
+                    acc[j][mt][i] += b;
+            }
+    }
+#pragma unroll
+    for(int mt = 0; mt < MT; mt++)
+    {
+        const int p = m_blk * BM + mt * 16 + r;
+        if(STAGE == 1)
+        {
+#pragma unroll
+            for(int j = 0; j < 2; j++)
+            {
+                float v[4];
+#pragma unroll
+                for(int i = 0; i < 4; i++)
+                    v[i] = ok[mt] ? silu_f32(acc[j][mt][i]) * acc[j + 2][mt][i] : 0.f;
+                uint2 o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                *(uint2*)(g.out + (size_t)p * I + nt * 128 + wave * 32 + j * 16 + kb * 4) = o;
+            }
+        }
+        else if(ok[mt])
+        {
+            const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
+            const float rw = g.sorted_w[p];
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+                uint2 o = make_uint2(pack_bf16x2(acc[j][mt][0] * rw, acc[j][mt][1] * rw),
+                                     pack_bf16x2(acc[j][mt][2] * rw, acc[j][mt][3] * rw));
+                *(uint2*)(g.out + ((size_t)tok * g.topk + slot) * g.N + nt * 256 + wave * 64 + j * 16 + kb * 4) = o;
+            }
+        }
+    }
+}
+
+template <int STAGE>
+static int launch_w4a16(const W4A16Args& g, int block_m, int64_t n_blk, hipStream_t stream)
+{
+    dim3 grid((unsigned)(n_blk * g.n_tiles)), block(W4A16_THREADS);
+    switch(block_m)
+    {
+    case 16: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1>), grid, block, 0, stream, g); break;
+    case 32: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2>), grid, block, 0, stream, g); break;
+    case 64: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4>), grid, block, 0, stream, g); break;
+    default: pyhip_set_error("moe_gemm_w4a16: block_m=%d not in {16,32,64}", block_m); return PYHIP_ERR_INVALID;
+    }
+    PYHIP_CHECK_LAUNCH("moe_gemm_w4a16_kernel");
+    return PYHIP_OK;
+}
+
+static int check_w4a16(const char* name, const void* a, const void* w, const void* w_s, const void* sorted_ids,
+                       const void* sorted_e, const void* num_valid, const void* out, int K, int block_m,
+                       int64_t n_blk, int64_t n_tiles)
+{
+    PYHIP_REQUIRE(a && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
+    PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64, "%s: block_m=%d not in {16,32,64}", name, block_m);
+    PYHIP_REQUIRE(n_blk >= 0 && n_blk * n_tiles < (1ll << 31), "%s: n_blk=%lld", name, (long long)n_blk);
+    PYHIP_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)w_s % 4) == 0 &&
+                      ((uintptr_t)out % 8) == 0,
+                  "%s: unaligned pointer", name);
+    return PYHIP_OK;
+}
+
+extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale,
+                                     const void* bias1_bf16, const uint32_t* sorted_ids,
+                                     const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* a2_bf16,
+                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                     int64_t n_blk, hipStream_t stream)
+{
+    int rc = check_w4a16("moe_gemm1_w4a16", hidden_bf16, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
+                         a2_bf16, hidden, block_m, n_blk, inter / 128);
+    if(rc)
+        return rc;
+    PYHIP_REQUIRE(inter > 0 && inter % 128 == 0, "moe_gemm1_w4a16: inter=%d must be a multiple of 128", inter);
+    PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0, "moe_gemm1_w4a16: bad sizes");
+    if(n_blk == 0)
+        return PYHIP_OK;
+    W4A16Args g;
+    g.a = (const uint16_t*)hidden_bf16; g.w = w1; g.w_s = w1_scale; g.bias = (const uint16_t*)bias1_bf16;
+    g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
+    g.out = (uint16_t*)a2_bf16; g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
+    g.SC = (hidden / 32 + 7) / 8 * 8; g.n_tiles = inter / 128;
+    return launch_w4a16<1>(g, block_m, n_blk, stream);
+}
+
+extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale,
+                                     const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
+                                     const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* out3_bf16,
+                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                     int64_t n_blk, hipStream_t stream)
+{
+    int rc = check_w4a16("moe_gemm2_w4a16", a2_bf16, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
+                         out3_bf16, inter, block_m, n_blk, hidden / 256);
+    if(rc)
+        return rc;
+    PYHIP_REQUIRE(sorted_weights, "moe_gemm2_w4a16: null sorted_weights");
+    PYHIP_REQUIRE(hidden > 0 && hidden % 256 == 0, "moe_gemm2_w4a16: hidden=%d must be a multiple of 256", hidden);
+    PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0, "moe_gemm2_w4a16: bad sizes");
+    if(n_blk == 0)
+        return PYHIP_OK;
+    W4A16Args g;
+    g.a = (const uint16_t*)a2_bf16; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
+    g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
+    g.num_valid = num_valid_ids; g.out = (uint16_t*)out3_bf16; g.T = tokens; g.topk = topk; g.K = inter;
+    g.N = hidden; g.SC = (inter / 32 + 7) / 8 * 8; g.n_tiles = hidden / 256;
+    return launch_w4a16<2>(g, block_m, n_blk, stream);
+}

@@ -6,8 +6,12 @@ and top-k ids in, per-token bf16 hidden states out.  Weights are MXFP4 (``quant_
 pre-shuffled layout, ``w1_scale`` / ``w2_scale`` e8m0 in the shuffled layout (see ``pyhip_amd.mxfp4``).
 
 Pipeline (all launches on the current torch stream, no host synchronisation):
-  sort -> quantise activations to MXFP4 -> gate_up GEMM + SiLU*up -> quantise -> down GEMM * routing
+  sort -> quantise activations to MXFP4 -> gate_up GEMM + SiLU*up (+ re-quantisation) -> down GEMM * routing
   weight -> top-k reduction.
+
+``method="w4a16"`` keeps the activations in bf16 (weights are expanded to bf16 in registers), the variant the
+reference runs for few tokens (src/contrib/moe.py:362-787); ``method="auto"`` is the MXFP4-activation path at
+every size.
 """
 import torch
 
@@ -119,7 +123,11 @@ def fused_moe(
 
     topk_ids = topk_ids.to(torch.int32).contiguous()
     topk_weight = topk_weight.to(torch.float32).contiguous()
+    assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
+    w4a16 = method == "w4a16"
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
+    if w4a16:
+        bm = min(bm, 64)
     ev = _mark("start")
     sorted_ids, sorted_w, sorted_e, num_valid, _, sched = moe_sorting(
         topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
@@ -134,6 +142,34 @@ def fused_moe(
     if bias2 is not None:
         bias2 = bias2.to(torch.bfloat16).contiguous()
         assert tuple(bias2.shape) == (E, H)
+
+    if w4a16:
+        hs = hidden_states.contiguous()
+        a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
+        rc = lib.pyhip_moe_gemm1_w4a16(_lib.dptr(hs), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(bias1),
+                                       _lib.dptr(sorted_ids), _lib.dptr(sorted_e), _lib.dptr(num_valid),
+                                       _lib.dptr(a2), T, k, global_E, H, I, bm, n_blk, stream)
+        _lib.check(rc, "moe_gemm1_w4a16")
+        ev = _mark("gemm1", ev)
+        out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
+        if expert_mask is not None or num_local_tokens is not None:
+            out3.zero_()
+        rc = lib.pyhip_moe_gemm2_w4a16(_lib.dptr(a2), _lib.dptr(w2u), _lib.dptr(w2s), _lib.dptr(bias2),
+                                       _lib.dptr(sorted_ids), _lib.dptr(sorted_w), _lib.dptr(sorted_e),
+                                       _lib.dptr(num_valid), _lib.dptr(out3), T, k, global_E, H, I, bm, n_blk, stream)
+        _lib.check(rc, "moe_gemm2_w4a16")
+        ev = _mark("gemm2", ev)
+        out = torch.empty(T, H, dtype=out_dtype, device=dev)
+        rc = lib.pyhip_moe_topk_reduce(_lib.dptr(out3), _lib.dptr(out), T, k, H,
+                                       1 if out_dtype == torch.float32 else 0, None, stream)
+        _lib.check(rc, "moe_topk_reduce")
+        _mark("reduce", ev)
+        if narrow:
+            out = out[:, : H - hidden_pad]
+        if return_parts:
+            return out, dict(sorted_ids=sorted_ids, sorted_weights=sorted_w, sorted_expert_ids=sorted_e,
+                             num_valid_ids=num_valid, a2=a2, out3=out3, block_m=bm)
+        return out
 
     a1_q, a1_s = act_quant_mxfp4(hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous())
     # the stage-1 kernel writes its result already quantised for stage 2; the bf16 copy is only produced on request
