@@ -99,7 +99,8 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     v4i wf[2][4];
     v4i af[2][MT][4];
     u32 wsc[4];                // scale dwords of the current 256-K column tile (two K-steps)
-    auto load_step = [&](int buf, int kt) __attribute__((always_inline)) {
+    auto load_step = [&](auto BB, int kt) __attribute__((always_inline)) {
+        constexpr int buf = decltype(BB)::value;
 #pragma unroll
         for(int j = 0; j < 4; j++)
             wf[buf][j] = __builtin_nontemporal_load((const v4i*)(wp[j] + (size_t)kt * 1024));
@@ -109,43 +110,37 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
             for(int i = 0; i < 4; i++)
                 af[buf][mt][i] = *(const v4i*)(ap[mt] + kt * 128 + i * 8);
     };
-    load_step(0, 0);
-    for(int kt = 0; kt < KT; kt++)
-    {
-        const int cur = kt & 1;
-        if((kt & 1) == 0)
+    // one K-step from register set P while the next one loads into set 1 - P (K / 128 is even)
+    auto k_step = [&](auto PP, int kt) __attribute__((always_inline)) {
+        constexpr int P = decltype(PP)::value;
+        if(P == 0)
         {
 #pragma unroll
             for(int j = 0; j < 4; j++)
                 wsc[j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
         }
         if(kt + 1 < KT)
-        {
-            if(cur == 0)
-                load_step(1, kt + 1);
-            else
-                load_step(0, kt + 1);
-        }
+            load_step(std::integral_constant<int, 1 - P>{}, kt + 1);
 #pragma unroll
         for(int j = 0; j < 4; j++)
         {
             // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
-            const u32 sb = (wsc[j] >> (8 * ((kt & 1) * 2 + sbyte_row[j]))) & 0xFFu;
+            const u32 sb = (wsc[j] >> (8 * (P * 2 + sbyte_row[j]))) & 0xFFu;
             v8bf wq[4];
-            if(cur == 0)
-                expand_fp4(wf[0][j], sb, wq);
-            else
-                expand_fp4(wf[1][j], sb, wq);
+            expand_fp4(wf[P][j], sb, wq);
 #pragma unroll
             for(int mt = 0; mt < MT; mt++)
 #pragma unroll
                 for(int i = 0; i < 4; i++)
-                {
-                    const v4i av = cur == 0 ? af[0][mt][i] : af[1][mt][i];
-                    acc[j][mt]   = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wq[i], __builtin_bit_cast(v8bf, av),
-                                                                         acc[j][mt], 0, 0, 0);
-                }
+                    acc[j][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wq[i], __builtin_bit_cast(v8bf, af[P][mt][i]),
+                                                                       acc[j][mt], 0, 0, 0);
         }
+    };
+    load_step(std::integral_constant<int, 0>{}, 0);
+    for(int kt = 0; kt < KT; kt += 2)
+    {
+        k_step(std::integral_constant<int, 0>{}, kt);
+        k_step(std::integral_constant<int, 1>{}, kt + 1);
     }
 
     // ---- epilogue: lane (r, kb) holds channels kb*4 .. kb*4+3 of row group j for token row r
