@@ -5,8 +5,9 @@ A step is one ``fused_moe`` call (sort -> quantise -> gate_up GEMM -> quantise -
 reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
 
   value     TFLOP/s of the whole layer at --tokens (default 8192), FLOPs = 6*T*k*I*H
-  decode    the same layer at --decode-tokens (default 16): ms, HBM GB/s on algorithmic bytes
-  decode_w4a16  the same with bf16 activations (method="w4a16")
+  decode    the same layer at --decode-tokens (default 16): ms, HBM GB/s on algorithmic bytes (method="auto":
+            bf16 activations x MXFP4 weights at this size)
+  decode_a4w4  the same with MXFP4 activations forced (method="a4w4")
   roofline  the dominant kernel (stage-1 gate_up GEMM) of the primary workload, timed with events
             recorded around it inside the timed steps
   cpu_baseline  the CPU oracle (oracle/moe.py) on a bounded sample of the same workload
@@ -127,7 +128,7 @@ def main():
     torch.cuda.synchronize()
     main_res = run_config(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m)
     dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
-    dec16 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), 0, "w4a16")
+    dec4 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
 
     if a.calibrate_copy:
         src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
@@ -162,16 +163,16 @@ def main():
                    "hbm_gbps": round(dec_gbps, 1), "frac_of_hbm_peak": round(dec_gbps / PEAK_HBM_GBPS, 4),
                    "tflops": round(dw["flops"] / (dec["ms"] * 1e-3) / 1e12, 2),
                    "stage_ms": {k: round(v, 4) for k, v in dec["stage_ms"].items()},
-                   "roofline": {"kernel": "moe_gemm_mxfp4_kernel<1,*> (gate_up)", "bound": "hbm",
+                   "roofline": {"kernel": "moe_gemm_w4a16_kernel<1,1> (gate_up, bf16 activations)", "bound": "hbm",
                                 "achieved": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                                 "unit": "GB/s",
                                 "frac": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                                 "traffic": None, "avg_launch_ms": round(dg1_ms, 4)}},
     }
-    out["decode_w4a16"] = {"tokens": a.decode_tokens, "ms_per_step": round(dec16["ms"], 4),
-                           "hbm_gbps": round(dw["bytes"] / (dec16["ms"] * 1e-3) / 1e9, 1),
-                           "frac_of_hbm_peak": round(dw["bytes"] / (dec16["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                           "stage_ms": {k: round(v, 4) for k, v in dec16["stage_ms"].items()}}
+    out["decode_a4w4"] = {"tokens": a.decode_tokens, "ms_per_step": round(dec4["ms"], 4),
+                          "hbm_gbps": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9, 1),
+                          "frac_of_hbm_peak": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                          "stage_ms": {k: round(v, 4) for k, v in dec4["stage_ms"].items()}}
     if a.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds)
     print(json.dumps(out))

@@ -10,8 +10,9 @@ Pipeline (all launches on the current torch stream, no host synchronisation):
   weight -> top-k reduction.
 
 ``method="w4a16"`` keeps the activations in bf16 (weights are expanded to bf16 in registers), the variant the
-reference runs for few tokens (src/contrib/moe.py:362-787); ``method="auto"`` is the MXFP4-activation path at
-every size.
+reference runs for few tokens (src/contrib/moe.py:362-787); ``method="a4w4"`` forces the MXFP4-activation path;
+``method="auto"`` takes w4a16 up to 4 routed rows per expert on average (where it is the faster of the two on
+MI355X and the layer is bound by weight streaming) and a4w4 above.
 """
 import torch
 
@@ -124,7 +125,9 @@ def fused_moe(
     topk_ids = topk_ids.to(torch.int32).contiguous()
     topk_weight = topk_weight.to(torch.float32).contiguous()
     assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
-    w4a16 = method == "w4a16"
+    # "auto" (and the reference's "jit" / "gluon", which name its own back ends): bf16 activations while the
+    # layer only streams weights (at most 4 routed rows per expert on average), MXFP4 activations above that
+    w4a16 = method == "w4a16" or (method != "a4w4" and T * k <= 4 * global_E)
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
     if w4a16:
         bm = min(bm, 64)

@@ -30,16 +30,17 @@ def _run(W, hidden, tw, ti, **kw):
     return fused_moe(hidden, W["w1"], W["w2"], tw, ti, w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], **kw)
 
 
-@pytest.mark.parametrize("T", [16, 1024, 8192])
-def test_sampled_experts_and_properties(layer, T):
+@pytest.mark.parametrize("T,method", [(16, "w4a16"), (16, "a4w4"), (1024, "a4w4"), (8192, "a4w4")])
+def test_sampled_experts_and_properties(layer, T, method):
     from pyhip_amd import mxfp4 as pm, workloads
     W = layer
     cfg = workloads.SHAPES[SHAPE]
     E, k, H, I = cfg["E"], cfg["k"], cfg["H"], cfg["I"]
     hidden, tw, ti = workloads.make_inputs(SHAPE, T)
-    print(f"full-size case {SHAPE} T={T}", flush=True)
-    out, parts = _run(W, hidden, tw, ti, return_parts=True)
-    out32 = _run(W, hidden, tw, ti, dtype=torch.float32)
+    print(f"full-size case {SHAPE} T={T} method={method}", flush=True)
+    a4 = method == "a4w4"
+    out, parts = _run(W, hidden, tw, ti, return_parts=True, method=method)
+    out32 = _run(W, hidden, tw, ti, dtype=torch.float32, method=method)
     torch.cuda.synchronize()
     out3 = parts["out3"]
     assert torch.isfinite(out.float()).all()
@@ -57,7 +58,7 @@ def test_sampled_experts_and_properties(layer, T):
     rng = np.random.default_rng(T)
     sample = rng.choice(hit, size=min(2, len(hit)), replace=False)
     x = hidden.float().cpu().numpy()
-    xq = moe.act_quant_dequant(x)
+    xq = moe.act_quant_dequant(x) if a4 else x
     twn = tw.cpu().numpy()
     for e in sample:
         e = int(e)
@@ -67,7 +68,7 @@ def test_sampled_experts_and_properties(layer, T):
                                  W["w2_scale_plain"][e * H:(e + 1) * H].cpu().numpy())
         t_idx, s_idx = np.nonzero(ids == e)
         a2 = moe.gateup_ref(xq[t_idx], w1)
-        ref = moe.down_ref(moe.act_quant_dequant(a2), w2, twn[t_idx, s_idx])
+        ref = moe.down_ref(moe.act_quant_dequant(a2) if a4 else a2, w2, twn[t_idx, s_idx])
         got = out3[torch.from_numpy(t_idx).cuda(), torch.from_numpy(s_idx).cuda()].float().cpu().numpy()
         rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
         err = np.abs(got - ref) - np.abs(ref) * 2.0 ** -7          # one bf16 ulp of the value
@@ -77,14 +78,14 @@ def test_sampled_experts_and_properties(layer, T):
 
     # (3) permuting the tokens permutes the output rows, bit for bit
     perm = torch.randperm(T, generator=torch.Generator().manual_seed(T)).cuda()
-    out_p = _run(W, hidden[perm].contiguous(), tw[perm].contiguous(), ti[perm].contiguous())
+    out_p = _run(W, hidden[perm].contiguous(), tw[perm].contiguous(), ti[perm].contiguous(), method=method)
     assert torch.equal(out_p, out[perm])
 
     # (4) routing weights times a power of two scale the output by exactly that factor
-    out_2 = _run(W, hidden, tw * 4.0, ti)
+    out_2 = _run(W, hidden, tw * 4.0, ti, method=method)
     assert torch.equal(out_2.float(), out.float() * 4.0)
 
     # (5) the order of a token's slots does not change what each (token, expert) pair produces
     rev = torch.arange(k - 1, -1, -1, device="cuda")
-    _, parts_r = _run(W, hidden, tw[:, rev].contiguous(), ti[:, rev].contiguous(), return_parts=True)
+    _, parts_r = _run(W, hidden, tw[:, rev].contiguous(), ti[:, rev].contiguous(), return_parts=True, method=method)
     assert torch.equal(parts_r["out3"][:, rev], out3)

@@ -133,9 +133,9 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
     b2 = None if L.bias2 is None else L.bias2.cuda()
     print(f"fused_moe case {name} T={T} bm={bm} bias={bias}", flush=True)
     out32, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
-                             bias1=b1, bias2=b2, dtype=torch.float32, return_parts=True)
+                             bias1=b1, bias2=b2, dtype=torch.float32, return_parts=True, method="a4w4")
     out16 = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
-                      bias1=b1, bias2=b2)
+                      bias1=b1, bias2=b2, method="a4w4")
     torch.cuda.synchronize()
     assert out16.dtype == torch.bfloat16 and out16.shape == (T, L.H)
 
@@ -180,7 +180,7 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
     print(f"padded case T={T} bm={bm} bias={bias}", flush=True)
     kw = dict(w1_scale=w1s, w2_scale=w2s, block_size_M=bm, bias1=b1, bias2=b2, hidden_pad=hp, intermediate_pad=ip,
-              dtype=torch.float32)
+              dtype=torch.float32, method="a4w4")
     out_narrow, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, return_parts=True, **kw)   # activations at the true width
     wide = torch.nn.functional.pad(L.hidden, (0, hp)).cuda()
     out_wide = fused_moe(wide, w1, w2, tw, ti, **kw)                                    # the reference's convention
@@ -237,3 +237,19 @@ def test_w4a16_matches_oracle(name, T, bm, bias):
     err, cos = metrics.max_err_over_rms(_f(out32), ref), metrics.cosine(_f(out32), ref)
     print(f"  max|err|/rms={err:.3e} (beyond the rounding allowance: {excess:.3e}) cosine={cos:.8f}", flush=True)
     assert excess <= TOL_MAX and cos >= TOL_COS
+
+
+def test_auto_dispatch():
+    """method="auto": bf16 activations up to 4 routed rows per expert on average, MXFP4 activations above"""
+    L = cases.make_layer("dsv3_s", 16, seed=2)            # 16 * 8 / 64 = 2 rows per expert
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s)
+    auto = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, **kw)
+    assert torch.equal(auto, fused_moe(L.hidden.cuda(), w1, w2, tw, ti, method="w4a16", **kw))
+    L = cases.make_layer("tiny", 64, seed=2)              # 64 * 2 / 8 = 16 rows per expert
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s)
+    auto = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, **kw)
+    assert torch.equal(auto, fused_moe(L.hidden.cuda(), w1, w2, tw, ti, method="a4w4", **kw))
