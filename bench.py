@@ -24,6 +24,14 @@ sys.path.insert(0, ROOT)
 PEAK_MFMA_FP4_TFLOPS = 10100.0     # MI355X dense MXFP4/MXFP6
 PEAK_HBM_GBPS = 8000.0
 
+# HBM-side bytes per launch of the gate_up GEMM, (shape, tokens) -> bytes, from the hardware counters
+# FETCH_SIZE (x 2.0: a plain 1 GiB device copy reads 524 288) + WRITE_SIZE (x 1.0), KiB per dispatch,
+# collected with `rocprofv3 --pmc` around this script; other workloads report null.
+MEASURED_TRAFFIC = {
+    ("dsv3", 8192): 3.713e6 * 2 * 1024 + 1.058e5 * 1024,
+    ("dsv3", 16): 8.012e5 * 2 * 1024 + 6.795e3 * 1024,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -158,7 +166,7 @@ def main():
         "stage_ms": {k: round(v, 4) for k, v in main_res["stage_ms"].items()},
         "roofline": {"kernel": "moe_gemm_mxfp4_kernel<1,*> (gate_up)", "bound": "mfma", "achieved": round(g1_tflops, 2),
                      "peak": PEAK_MFMA_FP4_TFLOPS, "unit": "TFLOP/s", "frac": round(g1_tflops / PEAK_MFMA_FP4_TFLOPS, 4),
-                     "traffic": None, "avg_launch_ms": round(g1_ms, 4)},
+                     "traffic": MEASURED_TRAFFIC.get((a.shape, a.tokens)), "avg_launch_ms": round(g1_ms, 4)},
         "decode": {"tokens": a.decode_tokens, "ms_per_step": round(dec["ms"], 4), "experts_hit": dw["e_hit"],
                    "hbm_gbps": round(dec_gbps, 1), "frac_of_hbm_peak": round(dec_gbps / PEAK_HBM_GBPS, 4),
                    "tflops": round(dw["flops"] / (dec["ms"] * 1e-3) / 1e12, 2),
@@ -167,7 +175,8 @@ def main():
                                 "achieved": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                                 "unit": "GB/s",
                                 "frac": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                                "traffic": None, "avg_launch_ms": round(dg1_ms, 4)}},
+                                "traffic": MEASURED_TRAFFIC.get((a.shape, a.decode_tokens)),
+                                "avg_launch_ms": round(dg1_ms, 4)}},
     }
     out["decode_a4w4"] = {"tokens": a.decode_tokens, "ms_per_step": round(dec4["ms"], 4),
                           "hbm_gbps": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9, 1),
