@@ -112,15 +112,18 @@ int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const ui
  * tests/contrib/moe/test_moe.py:347-374), the variant the reference uses when few tokens are routed.
  * Buffers as above, except hidden / a2 are bf16 ([tokens, hidden] in token order; [n_blk*block_m, inter] in
  * sorted-row order) and the down GEMM writes out3[tokens, topk, hidden] for pyhip_moe_topk_reduce instead of
- * adding into the layer output with atomics.  block_m is 16, 32 or 64; hidden % 512 == 0, inter % 512 == 0. */
+ * adding into the layer output with atomics.  block_m is 16, 32 or 64; hidden % 512 == 0, inter % 512 == 0.
+ * split_k: 4 = the four waves of a workgroup share a 64-row weight tile and split K between them (partial sums
+ * meet in LDS; four times as many workgroups), 1 = every wave owns 64 rows over the whole K, 0 = split when the
+ * launch would otherwise have fewer than 2048 workgroups with work. */
 int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale, const void* bias1_bf16,
                           const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
                           void* a2_bf16, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                          int64_t n_blk, pyhip_stream_t stream);
+                          int64_t n_blk, int split_k, pyhip_stream_t stream);
 int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale, const void* bias2_bf16,
                           const uint32_t* sorted_ids, const float* sorted_weights, const uint32_t* sorted_expert_ids,
                           const uint32_t* num_valid_ids, void* out3_bf16, int tokens, int topk, int experts,
-                          int hidden, int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
+                          int hidden, int inter, int block_m, int64_t n_blk, int split_k, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.

@@ -3,7 +3,12 @@
 // the bf16 MFMA.  This is the variant the reference runs when few tokens are routed
 // (src/contrib/moe.py:362-787, moe_2stage_splitk with fp4 weights, driven by
 // tests/contrib/moe/test_moe.py:347-374); at such sizes the layer only streams weights, so the kernel is kept
-// simple: one workgroup per (row block, weight tile), the K loop software-pipelined one K-step ahead, no LDS.
+// simple: one workgroup per (row block, weight tile), the K loop software-pipelined one K-step ahead.
+// Two mappings of a workgroup's four waves:
+//   SPLITK = false: tile of 256 weight rows, wave w owns 64 of them over the whole K range;
+//   SPLITK = true : tile of 64 weight rows shared by all waves, wave w takes K-steps w, w+4, ... and the four
+//                   partial sums meet in LDS (the reference's split-K arrangement, src/contrib/moe.py:362-500).
+//                   Four times as many workgroups: used when the layer would otherwise not fill the GPU.
 //
 // Operand mapping.  A pre-shuffled 1 KB weight block (src/misc.py:116-130) gives lane (row = l % 16,
 // kb = l / 16) the 32 consecutive K-elements kb*32 .. kb*32+31 of its row.  The bf16 MFMA 16x16x32 wants 8
@@ -46,10 +51,11 @@ __device__ __forceinline__ void expand_fp4(const v4i& w, u32 scale_byte, v8bf (&
 }
 
 // STAGE 1 = gate_up (+ SiLU(gate) * up), 2 = down (* routing weight).  MT = row groups of 16 per tile.
-template <int STAGE, int MT>
+template <int STAGE, int MT, bool SPLITK>
 __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
 {
     constexpr int BM = MT * 16;
+    __shared__ float red[SPLITK ? 4 * 4 * MT * WAVE * 4 : 1];      // [wave][j][mt][lane][4]
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int r = lane & 15, kb = lane >> 4;
@@ -58,6 +64,8 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
         return;
     const int e  = (int)g.sorted_e[m_blk];
     const int Kb = g.K / 2, I = g.N / 2;
+    // first output channel of this wave's rows (stage 1: within the gate half; the up half is I further)
+    const int chbase = STAGE == 1 ? (SPLITK ? nt * 32 : nt * 128 + wave * 32) : (SPLITK ? nt * 64 : nt * 256 + wave * 64);
 
     // weight row groups of this wave: j = 0..3 (stage 1: j>>1 selects gate / up)
     const uint8_t* wp[4];
@@ -67,8 +75,8 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
 #pragma unroll
     for(int j = 0; j < 4; j++)
     {
-        const size_t row = STAGE == 1 ? (size_t)e * g.N + (j >> 1) * I + nt * 128 + wave * 32 + (j & 1) * 16
-                                      : (size_t)e * g.N + nt * 256 + wave * 64 + j * 16;
+        const size_t row = STAGE == 1 ? (size_t)e * g.N + (j >> 1) * I + chbase + (j & 1) * 16
+                                      : (size_t)e * g.N + chbase + j * 16;
         wp[j]        = g.w + row * Kb + lane * 16;
         sp[j]        = g.w_s + (row / 32) * sc_tile + lane * 4;
         sbyte_row[j] = (int)((row / 16) & 1);
@@ -96,6 +104,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
             acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int KT = g.K / 128;
+    constexpr int KSTRIDE = SPLITK ? 4 : 1;
     v4i wf[2][4];
     v4i af[2][MT][4];
     u32 wsc[4];                // scale dwords of the current 256-K column tile (two K-steps)
@@ -113,19 +122,19 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     // one K-step from register set P while the next one loads into set 1 - P (K / 128 is even)
     auto k_step = [&](auto PP, int kt) __attribute__((always_inline)) {
         constexpr int P = decltype(PP)::value;
-        if(P == 0)
+        if(P == 0 || SPLITK)
         {
 #pragma unroll
             for(int j = 0; j < 4; j++)
                 wsc[j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
         }
-        if(kt + 1 < KT)
-            load_step(std::integral_constant<int, 1 - P>{}, kt + 1);
+        if(kt + KSTRIDE < KT)
+            load_step(std::integral_constant<int, 1 - P>{}, kt + KSTRIDE);
 #pragma unroll
         for(int j = 0; j < 4; j++)
         {
             // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
-            const u32 sb = (wsc[j] >> (8 * (P * 2 + sbyte_row[j]))) & 0xFFu;
+            const u32 sb = (wsc[j] >> (8 * ((kt & 1) * 2 + sbyte_row[j]))) & 0xFFu;
             v8bf wq[4];
             expand_fp4(wf[P][j], sb, wq);
 #pragma unroll
@@ -136,12 +145,40 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
                                                                        acc[j][mt], 0, 0, 0);
         }
     };
-    load_step(std::integral_constant<int, 0>{}, 0);
-    for(int kt = 0; kt < KT; kt += 2)
+    load_step(std::integral_constant<int, 0>{}, SPLITK ? wave : 0);
+    for(int kt = SPLITK ? wave : 0; kt < KT; kt += 2 * KSTRIDE)
     {
         k_step(std::integral_constant<int, 0>{}, kt);
-        k_step(std::integral_constant<int, 1>{}, kt + 1);
+        if(kt + KSTRIDE < KT)                                          // a wave's share of K-steps may be odd
+            k_step(std::integral_constant<int, 1>{}, kt + KSTRIDE);
     }
+    // which row groups this wave finishes: all four of its own, or (split K) the w-th of the shared ones
+    // (stage 1: gate group w and its up group w + 2, waves 0 and 1 only)
+    if(SPLITK)
+    {
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int mt = 0; mt < MT; mt++)
+                *(v4f*)&red[(((wave * 4 + j) * MT + mt) * WAVE + lane) * 4] = acc[j][mt];
+        __syncthreads();
+        if(STAGE == 1 && wave >= 2)
+            return;
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+#pragma unroll
+            for(int mt = 0; mt < MT; mt++)
+            {
+                v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for(int w = 0; w < 4; w++)
+                    sum += *(const v4f*)&red[(((w * 4 + j) * MT + mt) * WAVE + lane) * 4];
+                acc[j][mt] = sum;
+            }
+    }
+    auto mine = [&](int j) __attribute__((always_inline)) {
+        return !SPLITK || (STAGE == 1 ? (j & 1) == wave : j == wave);
+    };
 
     // ---- epilogue: lane (r, kb) holds channels kb*4 .. kb*4+3 of row group j for token row r
     if(g.bias)
@@ -151,8 +188,8 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
 #pragma unroll
             for(int i = 0; i < 4; i++)
             {
-                const int ch = STAGE == 1 ? (j >> 1) * I + nt * 128 + wave * 32 + (j & 1) * 16 + kb * 4 + i
-                                          : nt * 256 + wave * 64 + j * 16 + kb * 4 + i;
+                const int ch = STAGE == 1 ? (j >> 1) * I + chbase + (j & 1) * 16 + kb * 4 + i
+                                          : chbase + j * 16 + kb * 4 + i;
                 const float b = bf16_bits_to_f32(g.bias[(size_t)e * g.N + ch]);
 #pragma unroll
                 for(int mt = 0; mt < MT; mt++)
@@ -168,12 +205,14 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
 #pragma unroll
             for(int j = 0; j < 2; j++)
             {
+                if(!mine(j))
+                    continue;
                 float v[4];
 #pragma unroll
                 for(int i = 0; i < 4; i++)
                     v[i] = ok[mt] ? silu_f32(acc[j][mt][i]) * acc[j + 2][mt][i] : 0.f;
                 uint2 o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-                *(uint2*)(g.out + (size_t)p * I + nt * 128 + wave * 32 + j * 16 + kb * 4) = o;
+                *(uint2*)(g.out + (size_t)p * I + chbase + j * 16 + kb * 4) = o;
             }
         }
         else if(ok[mt])
@@ -183,23 +222,38 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
 #pragma unroll
             for(int j = 0; j < 4; j++)
             {
+                if(!mine(j))
+                    continue;
                 uint2 o = make_uint2(pack_bf16x2(acc[j][mt][0] * rw, acc[j][mt][1] * rw),
                                      pack_bf16x2(acc[j][mt][2] * rw, acc[j][mt][3] * rw));
-                *(uint2*)(g.out + ((size_t)tok * g.topk + slot) * g.N + nt * 256 + wave * 64 + j * 16 + kb * 4) = o;
+                *(uint2*)(g.out + ((size_t)tok * g.topk + slot) * g.N + chbase + j * 16 + kb * 4) = o;
             }
         }
     }
 }
 
+// split_k: 0 = decide here, 1 = never, 4 = always
 template <int STAGE>
-static int launch_w4a16(const W4A16Args& g, int block_m, int64_t n_blk, hipStream_t stream)
+static int launch_w4a16(W4A16Args g, int block_m, int64_t n_blk, int64_t rows, int experts, int split_k,
+                        hipStream_t stream)
 {
-    dim3 grid((unsigned)(n_blk * g.n_tiles)), block(W4A16_THREADS);
-    switch(block_m)
+    // upper bound of the row blocks that hold rows: one per routed row, and one partly filled block per expert
+    int64_t blocks = rows < n_blk ? rows : n_blk;
+    if(experts + rows / block_m < blocks)
+        blocks = experts + rows / block_m;
+    const bool split = split_k == 4 || (split_k == 0 && blocks * g.n_tiles < 2048);
+    if(split)
+        g.n_tiles *= 4;
+    // blocks past the bound cannot hold rows (the sort fills blocks from 0 upwards): no workgroups for them
+    dim3 grid((unsigned)(blocks * g.n_tiles)), block(W4A16_THREADS);
+    switch(block_m * 2 + (split ? 1 : 0))
     {
-    case 16: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1>), grid, block, 0, stream, g); break;
-    case 32: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2>), grid, block, 0, stream, g); break;
-    case 64: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4>), grid, block, 0, stream, g); break;
+    case 32: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1, false>), grid, block, 0, stream, g); break;
+    case 33: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1, true>), grid, block, 0, stream, g); break;
+    case 64: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2, false>), grid, block, 0, stream, g); break;
+    case 65: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2, true>), grid, block, 0, stream, g); break;
+    case 128: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4, false>), grid, block, 0, stream, g); break;
+    case 129: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4, true>), grid, block, 0, stream, g); break;
     default: pyhip_set_error("moe_gemm_w4a16: block_m=%d not in {16,32,64}", block_m); return PYHIP_ERR_INVALID;
     }
     PYHIP_CHECK_LAUNCH("moe_gemm_w4a16_kernel");
@@ -213,7 +267,7 @@ static int check_w4a16(const char* name, const void* a, const void* w, const voi
     PYHIP_REQUIRE(a && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
     PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
     PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64, "%s: block_m=%d not in {16,32,64}", name, block_m);
-    PYHIP_REQUIRE(n_blk >= 0 && n_blk * n_tiles < (1ll << 31), "%s: n_blk=%lld", name, (long long)n_blk);
+    PYHIP_REQUIRE(n_blk >= 0 && n_blk * n_tiles * 4 < (1ll << 31), "%s: n_blk=%lld", name, (long long)n_blk);
     PYHIP_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0 && ((uintptr_t)w_s % 4) == 0 &&
                       ((uintptr_t)out % 8) == 0,
                   "%s: unaligned pointer", name);
@@ -224,8 +278,9 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
                                      const void* bias1_bf16, const uint32_t* sorted_ids,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* a2_bf16,
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, hipStream_t stream)
+                                     int64_t n_blk, int split_k, hipStream_t stream)
 {
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4, "moe_gemm1_w4a16: split_k=%d not in {0,1,4}", split_k);
     int rc = check_w4a16("moe_gemm1_w4a16", hidden_bf16, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                          a2_bf16, hidden, block_m, n_blk, inter / 128);
     if(rc)
@@ -239,15 +294,16 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
     g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
     g.out = (uint16_t*)a2_bf16; g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
     g.SC = (hidden / 32 + 7) / 8 * 8; g.n_tiles = inter / 128;
-    return launch_w4a16<1>(g, block_m, n_blk, stream);
+    return launch_w4a16<1>(g, block_m, n_blk, (int64_t)tokens * topk, experts, split_k, stream);
 }
 
 extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale,
                                      const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* out3_bf16,
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, hipStream_t stream)
+                                     int64_t n_blk, int split_k, hipStream_t stream)
 {
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4, "moe_gemm2_w4a16: split_k=%d not in {0,1,4}", split_k);
     int rc = check_w4a16("moe_gemm2_w4a16", a2_bf16, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                          out3_bf16, inter, block_m, n_blk, hidden / 256);
     if(rc)
@@ -262,5 +318,5 @@ extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, con
     g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
     g.num_valid = num_valid_ids; g.out = (uint16_t*)out3_bf16; g.T = tokens; g.topk = topk; g.K = inter;
     g.N = hidden; g.SC = (inter / 32 + 7) / 8 * 8; g.n_tiles = hidden / 256;
-    return launch_w4a16<2>(g, block_m, n_blk, stream);
+    return launch_w4a16<2>(g, block_m, n_blk, (int64_t)tokens * topk, experts, split_k, stream);
 }

@@ -11,7 +11,7 @@ Pipeline (all launches on the current torch stream, no host synchronisation):
 
 ``method="w4a16"`` keeps the activations in bf16 (weights are expanded to bf16 in registers), the variant the
 reference runs for few tokens (src/contrib/moe.py:362-787); ``method="a4w4"`` forces the MXFP4-activation path;
-``method="auto"`` takes w4a16 up to 4 routed rows per expert on average (where it is the faster of the two on
+``method="auto"`` takes w4a16 up to 2 routed rows per expert on average (where it is the faster of the two on
 MI355X and the layer is bound by weight streaming) and a4w4 above.
 """
 import torch
@@ -87,7 +87,7 @@ def fused_moe(
     assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
     assert not doweight_stage1
     assert a1_scale is None and a2_scale is None, "activations are quantised dynamically"
-    assert splitk == 0
+    assert splitk in (0, 1, 4), "splitk: 0 = automatic, 1 = off, 4 = split K over the four waves (w4a16 path only)"
     assert w1_scale is not None and w2_scale is not None
     assert hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2
     out_dtype = hidden_states.dtype if dtype is None else dtype
@@ -126,8 +126,8 @@ def fused_moe(
     topk_weight = topk_weight.to(torch.float32).contiguous()
     assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
     # "auto" (and the reference's "jit" / "gluon", which name its own back ends): bf16 activations while the
-    # layer only streams weights (at most 4 routed rows per expert on average), MXFP4 activations above that
-    w4a16 = method == "w4a16" or (method != "a4w4" and T * k <= 4 * global_E)
+    # layer only streams weights (at most 2 routed rows per expert on average), MXFP4 activations above that
+    w4a16 = method == "w4a16" or (method != "a4w4" and T * k <= 2 * global_E)
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
     if w4a16:
         bm = min(bm, 64)
@@ -151,7 +151,7 @@ def fused_moe(
         a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
         rc = lib.pyhip_moe_gemm1_w4a16(_lib.dptr(hs), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(bias1),
                                        _lib.dptr(sorted_ids), _lib.dptr(sorted_e), _lib.dptr(num_valid),
-                                       _lib.dptr(a2), T, k, global_E, H, I, bm, n_blk, stream)
+                                       _lib.dptr(a2), T, k, global_E, H, I, bm, n_blk, splitk, stream)
         _lib.check(rc, "moe_gemm1_w4a16")
         ev = _mark("gemm1", ev)
         out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
@@ -159,7 +159,7 @@ def fused_moe(
             out3.zero_()
         rc = lib.pyhip_moe_gemm2_w4a16(_lib.dptr(a2), _lib.dptr(w2u), _lib.dptr(w2s), _lib.dptr(bias2),
                                        _lib.dptr(sorted_ids), _lib.dptr(sorted_w), _lib.dptr(sorted_e),
-                                       _lib.dptr(num_valid), _lib.dptr(out3), T, k, global_E, H, I, bm, n_blk, stream)
+                                       _lib.dptr(num_valid), _lib.dptr(out3), T, k, global_E, H, I, bm, n_blk, splitk, stream)
         _lib.check(rc, "moe_gemm2_w4a16")
         ev = _mark("gemm2", ev)
         out = torch.empty(T, H, dtype=out_dtype, device=dev)

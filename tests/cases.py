@@ -14,6 +14,7 @@ CONFIGS = {
     "dsv3_s": dict(E=64, k=8, H=1024, I=512, router="grouped"),
     # gpt-oss-shaped, scaled down: hidden = inter = 2880/2, not multiples of the kernels' 512-wide K tiles
     "gptoss_s": dict(E=16, k=4, H=1440, I=1440, router="softmax"),
+    "gptoss_s1": dict(E=16, k=4, H=1536, I=1536, router="softmax"),         # 12 K-steps: an odd share per wave under split K
 }
 
 

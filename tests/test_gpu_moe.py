@@ -199,11 +199,13 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     _end_to_end(_f(out_narrow), ref, ref_a2)
 
 
-@pytest.mark.parametrize("name,T,bm,bias", [
-    ("tiny", 64, 16, False), ("tiny", 5, 16, True), ("tiny", 200, 64, False), ("mixtral_s", 33, 32, False),
-    ("qwen3_s", 64, 16, False), ("dsv3_s", 16, None, False), ("dsv3_s", 128, None, True),
+@pytest.mark.parametrize("name,T,bm,bias,splitk", [
+    ("tiny", 64, 16, False, 1), ("tiny", 5, 16, True, 0), ("tiny", 200, 64, False, 1), ("mixtral_s", 33, 32, False, 1),
+    ("qwen3_s", 64, 16, False, 1), ("dsv3_s", 16, None, False, 1), ("dsv3_s", 128, None, True, 1),
+    ("tiny", 64, 16, True, 4), ("tiny", 200, 64, False, 4), ("mixtral_s", 33, 32, False, 4), ("dsv3_s", 16, None, False, 4),
+    ("gptoss_s1", 20, 16, True, 4),
 ])
-def test_w4a16_matches_oracle(name, T, bm, bias):
+def test_w4a16_matches_oracle(name, T, bm, bias, splitk):
     """bf16 activations x MXFP4 weights (method="w4a16") against the oracle's "a16" path:
     max|err| <= 1e-2 * rms(ref), cosine >= 0.999; the stage-1 result within one bf16 ulp."""
     L = cases.make_layer(name, T, seed=1, bias=bias)
@@ -211,9 +213,9 @@ def test_w4a16_matches_oracle(name, T, bm, bias):
     tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
     b1 = None if L.bias1 is None else L.bias1.cuda()
     b2 = None if L.bias2 is None else L.bias2.cuda()
-    print(f"w4a16 case {name} T={T} bm={bm} bias={bias}", flush=True)
+    print(f"w4a16 case {name} T={T} bm={bm} bias={bias} splitk={splitk}", flush=True)
     out32, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
-                             bias1=b1, bias2=b2, dtype=torch.float32, method="w4a16", return_parts=True)
+                             bias1=b1, bias2=b2, dtype=torch.float32, method="w4a16", return_parts=True, splitk=splitk)
     torch.cuda.synchronize()
     ref, a2_ref, slot_ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a16",
                                  bias1=None if L.bias1 is None else _f(L.bias1),
@@ -240,7 +242,7 @@ def test_w4a16_matches_oracle(name, T, bm, bias):
 
 
 def test_auto_dispatch():
-    """method="auto": bf16 activations up to 4 routed rows per expert on average, MXFP4 activations above"""
+    """method="auto": bf16 activations up to 2 routed rows per expert on average, MXFP4 activations above"""
     L = cases.make_layer("dsv3_s", 16, seed=2)            # 16 * 8 / 64 = 2 rows per expert
     w1, w1s, w2, w2s = cases.device_weights(L)
     tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
