@@ -255,3 +255,37 @@ def test_auto_dispatch():
     kw = dict(w1_scale=w1s, w2_scale=w2s)
     auto = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, **kw)
     assert torch.equal(auto, fused_moe(L.hidden.cuda(), w1, w2, tw, ti, method="a4w4", **kw))
+
+
+@pytest.mark.parametrize("name,T,method", [("dsv3_s", 16, "w4a16"), ("tiny", 300, "a4w4")])
+def test_graph_capture_replays(name, T, method):
+    """The whole layer is enqueue-only (no host synchronisation, no memset nodes), so it can be captured in a
+    HIP graph; every replay, with the inputs rewritten in place and eager work in between, must reproduce the
+    eager result bit for bit."""
+    L = cases.make_layer(name, T, seed=4)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    hidden = L.hidden.cuda()
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s, method=method)
+    print(f"graph case {name} T={T} method={method}", flush=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up outside the capture
+        fused_moe(hidden, w1, w2, tw, ti, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = fused_moe(hidden, w1, w2, tw, ti, **kw)
+    g = torch.Generator().manual_seed(11)
+    for rep in range(3):
+        hidden.copy_((torch.randn(T, L.H, generator=g)).to(torch.bfloat16))
+        perm = torch.randperm(T, generator=g)
+        ti.copy_(torch.from_numpy(L.topk_ids)[perm])    # a different routing on every replay
+        tw.copy_(torch.from_numpy(L.topk_w)[perm])
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out_g.clone()
+        eager = fused_moe(hidden, w1, w2, tw, ti, **kw)  # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), f"replay {rep}"
