@@ -125,8 +125,8 @@ def cpu_baseline(torch, W, shape, res, budget_s):
 def main():
     a = parse()
     if a.gpus != 1:
-        print("bench.py: this build runs on one GPU only (--gpus %d requested); expert-parallel sharding is "
-              "described in DESIGN.md but not built." % a.gpus, file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (--gpus %d requested); expert-parallel sharding over "
+              "several GPUs is not built." % a.gpus, file=sys.stderr)
         sys.exit(2)
     import torch
     from pyhip_amd import fused_moe, workloads

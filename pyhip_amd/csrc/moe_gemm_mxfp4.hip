@@ -42,10 +42,6 @@ struct GemmArgs
     uint8_t* out_s;            //          and its scales [n_blk*BM, OSK] in the activation-scale layout
     int OSK;
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
-#ifdef PYHIP_GEMM_DEBUG
-    int dbg;
-    unsigned long long* dbg_t;   // [gridDim][8] accumulated phase times (100 MHz ticks)
-#endif
 };
 
 // acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales; OPW / OPA select
@@ -491,13 +487,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
     };
 
     // ---------------------------------------------------------------- pipeline
-#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
-    unsigned long long tacc[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, t0 = wall_clock64(), t1;
-    const unsigned long long c_start = __builtin_readcyclecounter(), w_start = t0;
-#define TICK(i) do { t1 = wall_clock64(); tacc[i] += t1 - t0; t0 = t1; } while(0)
-#else
-#define TICK(i)
-#endif
     TileId cur, nxt;
     decode(cur);
     if(!cur.valid)
@@ -514,7 +503,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
     decode(nxt);                      // (without a schedule there is no next tile)
     zero_acc();
     int ks = 0;
-    TICK(0);                          // start-up
 
     // one K-group; returns false when the workgroup has no more work
     auto kgroup = [&](auto P) __attribute__((always_inline)) -> bool {
@@ -522,7 +510,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
         const bool last     = ks == KS - 1;
         const int kpre      = last ? 0 : ks + 1;  // K-group that is prefetched now (of the next tile when last)
         const int mb_nxt    = mb == 2 ? 0 : mb + 1;
-        TICK(1);                      // loop overhead since the last tick
         // (0) first K-group of a tile: ids/weights of the NEXT tile into the meta ring (two tiles ahead of the
         //     slot any wave can still be reading in its epilogue)
         // (1) descriptors of what this K-group prefetches: the next K-group of this tile, or K-group 0 of the
@@ -534,10 +521,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             else
                 setup_null();
         }
-#ifdef PYHIP_GEMM_DEBUG
-        if(g.dbg & 1) { wrs[0] = wrs[1] = make_rsrc(g.w, 0); wsrs[0] = wsrs[1] = make_rsrc(g.w_s, 0); }
-        if(g.dbg & 2) { ars = make_rsrc(g.a_q, 0); asrs = make_rsrc(g.a_s, 0); }
-#endif
         const bool meta_on = ks == 0 && nxt.valid;
         const v4i rid = make_rsrc(g.sorted_ids + (size_t)nxt.m_blk * BM, BM * 4);
         const v4i rwt = make_rsrc(g.sorted_w + (size_t)nxt.m_blk * BM, BM * 4);
@@ -571,7 +554,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                 vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], kpre * 512);
             }
         };
-        TICK(6);                      // tile bookkeeping
         __builtin_amdgcn_sched_barrier(0);
         static_for<4>([&](auto U) __attribute__((always_inline)) {
             constexpr int u = decltype(U)::value;
@@ -595,9 +577,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                     asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-#ifdef PYHIP_GEMM_DEBUG
-                if(!(g.dbg & 4))
-#endif
                 {
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
                 mfma_fp4<(u & 1) * 2 + 0, u>(acc[0][mt], wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
@@ -621,11 +600,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             // (4) weight tiles of the same K-step of the prefetched K-group into the registers just consumed
             load_wtiles(U, kpre * 4 + u);
             __builtin_amdgcn_sched_barrier(0);
-            TICK(7 + u);
         });
         // (5) the 16 weight loads above are the only VMEM ops younger than this group's DMAs
         wait_vmcnt_barrier<16>();
-        TICK(2);                      // wait + barrier
         ks++;
         if(last)
         {
@@ -633,10 +610,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             // first VALU read
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
             epilogue(cur, lds_meta[mb]);
-            TICK(3);
-#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
-            tacc[5] += 1;
-#endif
             if(!nxt.valid)
                 return false;
             cur = nxt;
@@ -644,7 +617,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             ks  = 0;
             zero_acc();
             decode(nxt);
-            TICK(4);
         }
         return true;
     };
@@ -655,25 +627,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
         if(!kgroup(std::integral_constant<int, 1>{}))
             break;
     }
-#if defined(PYHIP_GEMM_DEBUG) && PYHIP_GEMM_DEBUG > 1
-    if(g.dbg_t && threadIdx.x == 0)
-    {
-        tacc[1]  = __builtin_readcyclecounter() - c_start;   // shader clocks over the kernel
-        tacc[11] = wall_clock64() - w_start;                 // 100 MHz ticks over the kernel
-        for(int i = 0; i < 12; i++)
-            g.dbg_t[blockIdx.x * 12 + i] = tacc[i];
-    }
-#endif
 #endif
 }
 
 template <int STAGE>
 static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
 {
-#ifdef PYHIP_GEMM_DEBUG
-    g.dbg = getenv("PYHIP_DBG") ? atoi(getenv("PYHIP_DBG")) : 0;
-    g.dbg_t = getenv("PYHIP_DBG_T") ? (unsigned long long*)strtoull(getenv("PYHIP_DBG_T"), nullptr, 0) : nullptr;
-#endif
     unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
     if(g.K < 1024)
         g.sched = nullptr;   // a single K-group per tile: no room to prefetch across tiles, one tile per workgroup

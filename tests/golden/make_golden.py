@@ -10,7 +10,7 @@ Sources of the expected values:
   e2m1_ck.npz   float -> e2m1 codes of the reference's converter (archive/ck_tile/ck_tile/core/numeric/
                 mxfp_convert.hpp:61-216) for every tie and neighbourhood at several scales, the code -> float
                 table (pk_fp4.hpp:128-129) and the e8m0 byte -> float table (e8m0.hpp:85-100), same library
-  tiny_layer.npz  BASELINE config 0 (E=8, top-2, T=64, H=1024, I=512, seed 0): routing, checksums of the seeded
+  tiny_layer.npz  the tiny layer (E=8, top-2, T=64, H=1024, I=512, seed 0): routing, checksums of the seeded
                 inputs and the layer output of the CPU oracle (oracle/moe.py, act="a4").  A regression anchor
                 for the oracle and the known answer the GPU path is compared with.
 The fixtures are data only; no reference source is stored here.
@@ -75,7 +75,7 @@ def main():
     np.savez_compressed(os.path.join(HERE, "e2m1_ck.npz"), x_over_scale=xs, scales=scales, codes=codes,
                         e2m1_table=table, e8m0_table=e8)
 
-    # ---- config 0 layer
+    # ---- the tiny layer
     import cases as tc
     from oracle import moe
     L = tc.make_layer("tiny", 64, seed=0)

@@ -113,7 +113,7 @@ def _end_to_end(got32, ref, ref_given_a2):
 
 
 @pytest.mark.parametrize("name,T,bm,bias", [
-    ("tiny", 64, None, False),        # BASELINE config 0
+    ("tiny", 64, None, False),        # the tiny layer: E=8, top-2, T=64, H=1024, I=512
     ("tiny", 64, 16, False),
     ("tiny", 64, 32, True),
     ("tiny", 5, 16, False),
