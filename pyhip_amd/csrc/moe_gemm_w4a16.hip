@@ -134,7 +134,8 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
         for(int j = 0; j < 4; j++)
         {
             // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
-            const u32 sb = (wsc[j] >> (8 * ((kt & 1) * 2 + sbyte_row[j]))) & 0xFFu;
+            const int kpar = SPLITK ? (kt & 1) : P;          // without the split the parity is the register set
+            const u32 sb   = (wsc[j] >> (8 * (kpar * 2 + sbyte_row[j]))) & 0xFFu;
             v8bf wq[4];
             expand_fp4(wf[P][j], sb, wq);
 #pragma unroll

@@ -20,13 +20,21 @@ __global__ void __launch_bounds__(256)
         const int c       = (int)(id - t * H8);
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         const uint4* p = in + (t * k) * H8 + c;
-        for(int s = 0; s < k; s++)
+        for(int s0 = 0; s0 < k; s0 += 8)         // up to 8 independent loads in flight, added in slot order
         {
-            uint4 v = p[(long long)s * H8];
-            acc[0] += bf16_bits_to_f32(v.x & 0xFFFFu); acc[1] += bf16_bits_to_f32(v.x >> 16);
-            acc[2] += bf16_bits_to_f32(v.y & 0xFFFFu); acc[3] += bf16_bits_to_f32(v.y >> 16);
-            acc[4] += bf16_bits_to_f32(v.z & 0xFFFFu); acc[5] += bf16_bits_to_f32(v.z >> 16);
-            acc[6] += bf16_bits_to_f32(v.w & 0xFFFFu); acc[7] += bf16_bits_to_f32(v.w >> 16);
+            v4i v[8];
+#pragma unroll
+            for(int j = 0; j < 8; j++)
+                v[j] = s0 + j < k ? __builtin_nontemporal_load((const v4i*)(p + (long long)(s0 + j) * H8)) : (v4i){0, 0, 0, 0};
+#pragma unroll
+            for(int j = 0; j < 8; j++)
+            {
+                // (a slot past k adds +0.0, which leaves every value, including -0.0 sums, unchanged)
+                acc[0] += bf16_bits_to_f32((u32)v[j][0] & 0xFFFFu); acc[1] += bf16_bits_to_f32((u32)v[j][0] >> 16);
+                acc[2] += bf16_bits_to_f32((u32)v[j][1] & 0xFFFFu); acc[3] += bf16_bits_to_f32((u32)v[j][1] >> 16);
+                acc[4] += bf16_bits_to_f32((u32)v[j][2] & 0xFFFFu); acc[5] += bf16_bits_to_f32((u32)v[j][2] >> 16);
+                acc[6] += bf16_bits_to_f32((u32)v[j][3] & 0xFFFFu); acc[7] += bf16_bits_to_f32((u32)v[j][3] >> 16);
+            }
         }
         if(OUT_F32)
         {
