@@ -84,7 +84,7 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
  *                tests/contrib/moe/test_moe.py:732-744.  Needs inter % 512 == 0.  At least one of a2 and
  *                a2_q must be given.
  * block_m must equal the block_size the sort ran with and `experts` the expert count it ran with;
- * block_m is 16, 32, 64 or 128; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
+ * block_m is 16, 32, 64, 128 or 256; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
  * workgroup per tile and worst-case block is launched, as the reference does). */
 int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,

@@ -56,6 +56,34 @@ __device__ __forceinline__ void mfma_fp4(v4f& acc, v4i w, v4i a, int w_scale, in
                  : "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1), "n"(OPW >> 1), "n"(OPA >> 1));
 }
 
+// The same with the accumulator in the accumulation registers a[ACC0 .. ACC0+3], named in the instruction text:
+// the compiler never sees these registers as values.  Tiles of 256 rows need 256 accumulator registers per lane
+// on top of the operand registers; declared as ordinary vectors (in either register file) the compiler keeps
+// shuffling them between the files around the loop and spills.  With the register numbers fixed by hand, the
+// kernel reserves all 256 accumulation registers once (see the clobber at its top) and must keep its ordinary
+// register use below the point where the compiler would start parking values in them (checked at build time by
+// looking for accumulation-register moves outside these helpers).
+template <int OPW, int OPA, int ACC0>
+__device__ __forceinline__ void mfma_fp4_fixed(v4i w, v4i a, int w_scale, int a_scale)
+{
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0] cbsz:4 blgp:4"
+                 :
+                 : "n"(ACC0), "n"(ACC0 + 3), "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1),
+                   "n"(OPW >> 1), "n"(OPA >> 1));
+}
+template <int R>
+__device__ __forceinline__ float acc_fixed_read()
+{
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(R));
+    return x;
+}
+template <int R>
+__device__ __forceinline__ void acc_fixed_zero()
+{
+    asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(R));
+}
+
 // ---- vector-memory primitives.  Every VMEM operation of the pipeline is issued through inline assembly
 // and every wait on the VMEM counter is written by hand: the counter retires loads in issue order, the
 // issue order below is fixed, so "all but the N youngest operations have completed" is exact.  (Left to
@@ -147,10 +175,13 @@ struct TileId
 // a tile boundary needs (schedule tables, sorted ids, routing weights) is read from LDS, so no wait on the
 // vector-memory counter ever covers the prefetches in flight.
 template <int STAGE, int MT>
-__global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArgs g)
+__global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     constexpr int BM    = MT * 16;
+    constexpr bool ACC_FIXED = MT > 8;        // accumulators in hand-numbered accumulation registers (256-row tiles)
+    if constexpr(ACC_FIXED)
+        asm volatile("" ::: "a0", "a255");    // reserves a0 .. a255 for this kernel
     constexpr int NA    = (MT + 3) / 4;       // activation row groups DMA'd per wave
     constexpr int SLOTS = NA * 4;             // row-group slots per LDS stage (slots >= MT are never read)
     constexpr int NID   = (BM + 63) / 64;     // DMA ops that bring one tile's sorted ids (same for weights)
@@ -357,13 +388,38 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             vm_load_b128<0>(wf[u][j], w_voff[j & 1] + (j >> 1) * w_half, wrs[j >> 1], kt * 1024);
     };
 
-    v4f acc[4][MT];
+    // accumulator of (weight row group j, row group mt): acc[j][mt], or a[(j*MT + mt)*4 .. +3] when ACC_FIXED
+    v4f acc[4][ACC_FIXED ? 1 : MT];
     auto zero_acc = [&]() __attribute__((always_inline)) {
+        if constexpr(ACC_FIXED)
+            static_for<16 * MT>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
+        else
+        {
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+            for(int j = 0; j < 4; j++)
 #pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-                acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+                for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
+                    acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // the four accumulators of row group MTI (plus bias, when ACC_FIXED: there the bias is added here instead of
+    // being folded into the accumulators first)
+    auto fetch_row = [&](auto MTI, v4f (&row)[4], const float (&bz)[4][4]) __attribute__((always_inline)) {
+        constexpr int mt = decltype(MTI)::value;
+        if constexpr(ACC_FIXED)
+        {
+            static_for<4>([&](auto J) __attribute__((always_inline)) {
+                constexpr int j = decltype(J)::value, a0 = (j * MT + mt) * 4;
+                row[j] = (v4f){acc_fixed_read<a0>() + bz[j][0], acc_fixed_read<a0 + 1>() + bz[j][1],
+                               acc_fixed_read<a0 + 2>() + bz[j][2], acc_fixed_read<a0 + 3>() + bz[j][3]};
+            });
+        }
+        else
+        {
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+                row[j] = acc[j][ACC_FIXED ? 0 : mt];
+        }
     };
 
     // ---------------------------------------------------------------- epilogue of one tile
@@ -375,27 +431,31 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             typedef unsigned v2u __attribute__((ext_vector_type(2)));
             uint16_t* out = (uint16_t*)g.out;
             const int chw = t.nt * 128 + wave * 32;
+            float bz[4][4] = {};
             if(g.bias)      // rare: fold the biases into the accumulators first
             {
 #pragma unroll
                 for(int j = 0; j < 4; j++)
                 {
-                    float b[4];
 #pragma unroll
                     for(int i = 0; i < 4; i++)
-                        b[i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4 + i]);
+                        bz[j][i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4 + i]);
+                    if constexpr(!ACC_FIXED)
+                    {
 #pragma unroll
-                    for(int mt = 0; mt < MT; mt++)
+                        for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
 #pragma unroll
-                        for(int i = 0; i < 4; i++)
-                            acc[j][mt][i] += b[i];
+                            for(int i = 0; i < 4; i++)
+                                acc[j][mt][i] += bz[j][i];
+                    }
                 }
             }
             // after the swap: lane rows 0..3 hold channel offsets 0, 16, 8, 24
             const int ch_out = chw + (kb & 1) * 16 + (kb >> 1) * 8;
-#pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-            {
+            static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
+                constexpr int mt = decltype(MTI)::value;
+                v4f row[4];
+                fetch_row(MTI, row, bz);
                 const int p   = t.m_blk * BM + mt * 16 + r;
                 const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
                 u32 d[2][2];
@@ -405,7 +465,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                     float v[4];
 #pragma unroll
                     for(int i = 0; i < 4; i++)
-                        v[i] = ok ? silu_f32(acc[j][mt][i]) * acc[j + 2][mt][i] : 0.f;
+                        v[i] = ok ? silu_f32(row[j][i]) * row[j + 2][i] : 0.f;
                     d[j][0] = pack_bf16x2(v[0], v[1]);
                     d[j][1] = pack_bf16x2(v[2], v[3]);
                 }
@@ -434,7 +494,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
-            }
+            });
         }
         else
         {
@@ -442,25 +502,29 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             // four lane rows gives every lane 16 consecutive channels: 32 B stores, 128 B contiguous per row.
             uint16_t* out = (uint16_t*)g.out;
             const int chw = t.nt * 256 + wave * 64;
+            float bz[4][4] = {};
             if(g.bias)      // rare: fold the bias into the accumulators first
             {
 #pragma unroll
                 for(int j = 0; j < 4; j++)
                 {
-                    float b[4];
 #pragma unroll
                     for(int i = 0; i < 4; i++)
-                        b[i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + chw + j * 16 + kb * 4 + i]);
+                        bz[j][i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + chw + j * 16 + kb * 4 + i]);
+                    if constexpr(!ACC_FIXED)
+                    {
 #pragma unroll
-                    for(int mt = 0; mt < MT; mt++)
+                        for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
 #pragma unroll
-                        for(int i = 0; i < 4; i++)
-                            acc[j][mt][i] += b[i];
+                            for(int i = 0; i < 4; i++)
+                                acc[j][mt][i] += bz[j][i];
+                    }
                 }
             }
-#pragma unroll
-            for(int mt = 0; mt < MT; mt++)
-            {
+            static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
+                constexpr int mt = decltype(MTI)::value;
+                v4f row[4];
+                fetch_row(MTI, row, bz);
                 const u32 id   = meta[mt * 16 + r];
                 const float rw = __builtin_bit_cast(float, meta[MPAD + mt * 16 + r]);
                 const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
@@ -469,8 +533,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
 #pragma unroll
                 for(int j = 0; j < 4; j++)
                 {
-                    lo[j] = pack_bf16x2(acc[j][mt][0] * rw, acc[j][mt][1] * rw);
-                    hi[j] = pack_bf16x2(acc[j][mt][2] * rw, acc[j][mt][3] * rw);
+                    lo[j] = pack_bf16x2(row[j][0] * rw, row[j][1] * rw);
+                    hi[j] = pack_bf16x2(row[j][2] * rw, row[j][3] * rw);
                 }
                 transpose4x4_rows(lo);
                 transpose4x4_rows(hi);
@@ -482,7 +546,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                     dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
                 }
                 __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
-            }
+            });
         }
     };
 
@@ -554,6 +618,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                 vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], kpre * 512);
             }
         };
+        constexpr int RA = 4;
+        v4i af_r[RA + 1];
+        int asc_all[ACC_FIXED ? MT : 1];         // the scale dword of a row group serves all four K-steps
+        auto lds_read = [&](auto NN) __attribute__((always_inline)) {
+            constexpr int n = decltype(NN)::value, uu = n / MT, mm = n % MT;
+            af_r[n % (RA + 1)] = *(const v4i*)(stage[p] + (uu * SLOTS + mm) * 1024 + rd_a);
+            if constexpr(uu == 0)
+                asc_all[ACC_FIXED ? mm : 0] = *(const int*)(sstage[p] + mm * 256 + rd_s);
+        };
+        if constexpr(ACC_FIXED)
+            static_for<RA>([&](auto NN) __attribute__((always_inline)) { lds_read(NN); });
         __builtin_amdgcn_sched_barrier(0);
         static_for<4>([&](auto U) __attribute__((always_inline)) {
             constexpr int u = decltype(U)::value;
@@ -564,14 +639,29 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
             if(u == 0)
                 wait_vm_scales<YOUNGER>(w_sc[p][0], w_sc[p][1], w_sc[p][2], w_sc[p][3]);
             // activation operand and its scale dword (one per 16-row group and K-group, op_sel picks this K-step's
-            // byte) are read one row group ahead of the MFMAs that consume them
-            v4i af  = *(const v4i*)(stage[p] + (u * SLOTS) * 1024 + rd_a);
-            int asc = *(const int*)(sstage[p] + rd_s);
+            // byte) are read ahead of the MFMAs that consume them: one row group ahead within a K-step with two
+            // waves per SIMD, RA row groups ahead across K-step boundaries (a ring of RA + 1 register sets) in
+            // the one-wave-per-SIMD 256-row tile, where nothing else covers the LDS latency
+            v4i af  = {0, 0, 0, 0};
+            int asc = 0;
+            if constexpr(!ACC_FIXED)
+            {
+                af  = *(const v4i*)(stage[p] + (u * SLOTS) * 1024 + rd_a);
+                asc = *(const int*)(sstage[p] + rd_s);
+            }
             static_for<MT>([&](auto M) __attribute__((always_inline)) {
                 constexpr int mt = decltype(M)::value;
                 v4i af_n  = af;
                 int asc_n = asc;
-                if constexpr(mt + 1 < MT)
+                if constexpr(ACC_FIXED)
+                {
+                    constexpr int n = u * MT + mt;             // position in the K-group's sequence of row groups
+                    if constexpr(n + RA < 4 * MT)
+                        lds_read(std::integral_constant<int, n + RA>{});
+                    af  = af_r[n % (RA + 1)];
+                    asc = asc_all[ACC_FIXED ? mt : 0];
+                }
+                else if constexpr(mt + 1 < MT)
                 {
                     af_n  = *(const v4i*)(stage[p] + (u * SLOTS + mt + 1) * 1024 + rd_a);
                     asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
@@ -579,10 +669,21 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                 __builtin_amdgcn_sched_barrier(0);
                 {
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                mfma_fp4<(u & 1) * 2 + 0, u>(acc[0][mt], wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
-                mfma_fp4<(u & 1) * 2 + 1, u>(acc[1][mt], wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
-                mfma_fp4<(u & 1) * 2 + 0, u>(acc[2][mt], wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
-                mfma_fp4<(u & 1) * 2 + 1, u>(acc[3][mt], wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
+                if constexpr(ACC_FIXED)
+                {
+                    mfma_fp4_fixed<(u & 1) * 2 + 0, u, (0 * MT + mt) * 4>(wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
+                    mfma_fp4_fixed<(u & 1) * 2 + 1, u, (1 * MT + mt) * 4>(wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
+                    mfma_fp4_fixed<(u & 1) * 2 + 0, u, (2 * MT + mt) * 4>(wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
+                    mfma_fp4_fixed<(u & 1) * 2 + 1, u, (3 * MT + mt) * 4>(wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
+                }
+                else
+                {
+                    constexpr int am = ACC_FIXED ? 0 : mt;
+                    mfma_fp4<(u & 1) * 2 + 0, u>(acc[0][am], wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
+                    mfma_fp4<(u & 1) * 2 + 1, u>(acc[1][am], wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
+                    mfma_fp4<(u & 1) * 2 + 0, u>(acc[2][am], wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
+                    mfma_fp4<(u & 1) * 2 + 1, u>(acc[3][am], wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
+                }
                 }
                 // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
                 // issue overlaps the matrix pipeline instead of preceding it
@@ -593,8 +694,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, 2) moe_gemm_mxfp4_kernel(GemmArg
                             prefetch_op(std::integral_constant<int, k>{});
                     });
                 __builtin_amdgcn_sched_barrier(0);
-                af  = af_n;
-                asc = asc_n;
+                if constexpr(!ACC_FIXED)
+                {
+                    af  = af_n;
+                    asc = asc_n;
+                }
             });
             __builtin_amdgcn_sched_barrier(0);
             // (4) weight tiles of the same K-step of the prefetched K-group into the registers just consumed
@@ -642,7 +746,7 @@ static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
         int dev = 0, cus = 256;
         if(hipGetDevice(&dev) == hipSuccess)
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        unsigned resident = (unsigned)cus * 2u / 8u * 8u;
+        unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
     dim3 grid(nwg), block(GEMM_THREADS);
@@ -652,7 +756,8 @@ static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
     case 32: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 2>), grid, block, 0, stream, g); break;
     case 64: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 4>), grid, block, 0, stream, g); break;
     case 128: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 8>), grid, block, 0, stream, g); break;
-    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128}", block_m); return PYHIP_ERR_INVALID;
+    case 256: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 16>), grid, block, 0, stream, g); break;
+    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256}", block_m); return PYHIP_ERR_INVALID;
     }
     PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel");
     return PYHIP_OK;
@@ -664,8 +769,8 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 {
     PYHIP_REQUIRE(a_q && a_s && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
     PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
-    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128,
-                  "%s: block_m=%d not in {16,32,64,128}", name, block_m);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256,
+                  "%s: block_m=%d not in {16,32,64,128,256}", name, block_m);
     PYHIP_REQUIRE(n_blk >= 0 && n_blk < (1 << 24), "%s: n_blk=%lld", name, (long long)n_blk);
     PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < (1ll << 32),
                   "%s: activation matrix of %lld rows x %d exceeds the 4 GiB buffer range", name, (long long)a_rows, K);

@@ -119,6 +119,8 @@ def _end_to_end(got32, ref, ref_given_a2):
     ("tiny", 5, 16, False),
     ("tiny", 300, 64, False),
     ("tiny", 300, 128, True),
+    ("tiny", 300, 256, True),         # 256-row tile: accumulators in hand-numbered accumulation registers
+    ("mixtral_s", 700, 256, False),
     ("mixtral_s", 33, 32, False),
     ("qwen3_s", 64, 16, False),
     ("qwen3_s", 257, 64, False),
