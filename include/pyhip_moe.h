@@ -26,6 +26,23 @@ int pyhip_moe_abi_version(void);
 const char* pyhip_moe_last_error(void);
 
 /* ------------------------------------------------------------------------------------------
+ * Routers: gating scores f32 [tokens, experts] -> topk_weight f32 [tokens, topk], topk_ids i32 [tokens, topk],
+ * the inputs of the routing sort.  Picks are in descending score order; ties go to the lower expert index.
+ * experts must be 64 * 2^n, at most 2048 (pad the scores with -inf columns otherwise); topk <= 64.
+ *   pyhip_moe_topk_softmax          softmax over the experts, top-k, weights renormalised to sum 1 when
+ *                                   renormalize != 0: replaces aiter.fused_topk(hidden, score, topk, True) as
+ *                                   called at tests/contrib/moe/test_fused_moe.py:38,87.
+ *   pyhip_moe_topk_grouped_sigmoid  DeepSeek-V3 routing: sigmoid scores, the experts form n_group equal groups
+ *                                   of consecutive experts, the topk_group groups with the largest sum of their
+ *                                   two best scores stay, top-k inside them.  Not in the reference (its tests
+ *                                   draw ids with torch.topk(randn), tests/contrib/moe/test_moe_sorting.py:81-84);
+ *                                   n_group must be a power of two <= 64. */
+int pyhip_moe_topk_softmax(const float* gating, int tokens, int experts, int topk, int renormalize,
+                           float* topk_weight, int32_t* topk_ids, pyhip_stream_t stream);
+int pyhip_moe_topk_grouped_sigmoid(const float* gating, int tokens, int experts, int topk, int n_group, int topk_group,
+                                   int renormalize, float* topk_weight, int32_t* topk_ids, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * Routing sort.  Replaces aiter.fused_moe.moe_sorting as called at src/contrib/fused_moe.py:283,
  * 301-305,368-372 (CPU statement of the result: src/contrib/fused_moe.py:56-100; in-tree C++
  * statement: archive/ck_tile/ck_tile/host/reference/reference_moe_sorting.hpp:13-117) and the

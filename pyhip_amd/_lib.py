@@ -15,6 +15,8 @@ _P, _I, _L = _c.c_void_p, _c.c_int, _c.c_int64
 SIGNATURES = {
     "pyhip_moe_abi_version": (_I, []),
     "pyhip_moe_last_error": (_c.c_char_p, []),
+    "pyhip_moe_topk_softmax": (_I, [_P, _I, _I, _I, _I, _P, _P, _P]),
+    "pyhip_moe_topk_grouped_sigmoid": (_I, [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P]),
     "pyhip_moe_sorting_max_blocks": (_L, [_L, _I, _I, _I]),
     "pyhip_moe_sorting_workspace_bytes": (_L, [_L, _I, _I]),
     "pyhip_moe_schedule_words": (_L, [_I]),
