@@ -14,7 +14,10 @@ LIB = os.path.join(HERE, "libpyhip_moe.so")
 SOURCES = ["capi.hip", "moe_sort.hip", "moe_quant.hip", "moe_gemm_mxfp4.hip", "moe_gemm_w4a16.hip", "moe_reduce.hip", "moe_router.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # the GEMM keeps its accumulators in hand-numbered accumulation registers: the compiler must not park
+         # spilled values there
+         "-mllvm", "-amdgpu-spill-vgpr-to-agpr=0"]
 
 
 def _run(cmd):

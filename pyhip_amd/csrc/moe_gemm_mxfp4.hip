@@ -179,9 +179,15 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     constexpr int BM    = MT * 16;
-    constexpr bool ACC_FIXED = MT > 8;        // accumulators in hand-numbered accumulation registers (256-row tiles)
-    if constexpr(ACC_FIXED)
-        asm volatile("" ::: "a0", "a255");    // reserves a0 .. a255 for this kernel
+    // The accumulators live in the accumulation registers a0 .. a[16*MT-1], named by hand in the instruction text
+    // (mfma_fp4_fixed); the clobber reserves that range for the kernel.  RING: the one-wave-per-SIMD 256-row tile
+    // reads its LDS operands through a deeper ring of registers.
+    constexpr bool RING = MT > 8;
+    if constexpr(MT == 16) asm volatile("" ::: "a0", "a255");
+    if constexpr(MT == 8) asm volatile("" ::: "a0", "a127");
+    if constexpr(MT == 4) asm volatile("" ::: "a0", "a63");
+    if constexpr(MT == 2) asm volatile("" ::: "a0", "a31");
+    if constexpr(MT == 1) asm volatile("" ::: "a0", "a15");
     constexpr int NA    = (MT + 3) / 4;       // activation row groups DMA'd per wave
     constexpr int SLOTS = NA * 4;             // row-group slots per LDS stage (slots >= MT are never read)
     constexpr int NID   = (BM + 63) / 64;     // DMA ops that bring one tile's sorted ids (same for weights)
@@ -192,7 +198,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // A weight tile loaded after K-step u is consumed by K-step u of the next K-group; younger than it at
     // that point are the tiles of the later K-steps, and for u > 0 this K-group's prefetches and tiles.
     constexpr int NPF = NM + 5 * NA + 4;
-    constexpr int PPM = (NPF + MT - 1) / MT;   // prefetch operations issued after each row group's MFMAs
     // one LDS stage = the activation tile of a whole K-group (4 K-steps of 128) + its scales
     __shared__ __attribute__((aligned(16))) uint8_t lds_a0[4 * SLOTS * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t lds_a1[4 * SLOTS * 1024];
@@ -308,6 +313,19 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         ars  = make_rsrc(g.a_q, 0);
         asrs = make_rsrc(g.a_s, 0);
     };
+    // Row groups of a tile that hold at least one real row.  The sort pads every expert's rows at the END of
+    // its last block, so the real rows of a block are a prefix: padded row groups are skipped by the MFMA loop
+    // (kgroup<.., MA>) and their activation fetches are sent out of the descriptor's range, where the
+    // hardware drops them.  Rounded up to the granularity the K-group body is instantiated for.
+    constexpr int MA_STEP = MT > 8 ? 2 : MT;
+    constexpr u32 OOB     = 0xFFFF0000u;           // beyond every activation buffer (checked by the launcher)
+    auto count_groups = [&](const u32* ids) __attribute__((always_inline)) -> int {
+        const u32 id  = ids[(lane < MT ? lane : 0) * 16];
+        const bool ok = lane < MT && (int)(id >> 24) < g.topk && (int)(id & 0xFFFFFFu) < g.T;
+        int n         = __builtin_popcountll(__ballot(ok));
+        n             = n < 1 ? 1 : n;
+        return (n + MA_STEP - 1) / MA_STEP * MA_STEP;
+    };
     // ids: the tile's sorted ids, either in LDS (meta buffer) or in global memory
     auto setup_load = [&](const TileId& t, const u32* ids) __attribute__((always_inline)) {
         const size_t sc_tile = (size_t)(g.SC / 8) * 256;           // bytes of one 32-row scale tile
@@ -333,20 +351,16 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         for(int i = 0; i < NA; i++)
         {
             const int slot = wave + 4 * i;
-            int row        = 0;                      // padding rows and unused slots read row 0; never stored
+            int row        = -1;                     // padding rows and unused slots fetch nothing
             if(slot < MT)
             {
-                if(STAGE == 1)
-                {
-                    const u32 id  = ids[slot * 16 + dma_row];
-                    const int tok = (int)(id & 0xFFFFFFu);
-                    row           = ((int)(id >> 24) < g.topk && tok < g.T) ? tok : 0;
-                }
-                else
-                    row = t.m_blk * BM + slot * 16 + dma_row;
+                const u32 id  = ids[slot * 16 + dma_row];
+                const int tok = (int)(id & 0xFFFFFFu);
+                if((int)(id >> 24) < g.topk && tok < g.T)
+                    row = STAGE == 1 ? tok : t.m_blk * BM + slot * 16 + dma_row;
             }
-            a_off[i]  = row * Kb + dma_chunk * 16;
-            as_off[i] = row * g.SK + (lane & 3) * 4;
+            a_off[i]  = row < 0 ? (int)OOB : row * Kb + dma_chunk * 16;
+            as_off[i] = row < 0 ? (int)OOB : row * g.SK + (lane & 3) * 4;
         }
     };
 
@@ -369,8 +383,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     };
     v4i wf[4][4];
     int w_sc[2][4];
-    // per-lane offsets of the wave's row groups inside wrs[] / of its scale dwords inside wsrs[]
-    const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1 (+32*Kb for stage 2, h = 1)
+    // per-lane offsets of the wave's row groups inside wrs[] / of its scale dwords inside wsrs[]; the half that
+    // is uniform (stage 2: row groups 2, 3 sit 32 rows further in the same descriptor) goes into the scalar offset,
+    // which the hardware does not range-check: it stays inside the rows the descriptor covers
+    const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1
     const int w_half     = (STAGE == 2) ? 32 * Kb : 0;
     const int ws_half    = (STAGE == 2) ? (g.SC / 8) * 256 : 0;
     auto load_wscales = [&](auto S, int ks) __attribute__((always_inline)) {
@@ -379,51 +395,39 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         for(int h = 0; h < 2; h++)
 #pragma unroll
             for(int c = 0; c < 2; c++)
-                vm_load_b32<0>(w_sc[s][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], ks * 512);
+                vm_load_b32<0>(w_sc[s][h * 2 + c], lane * 4 + c * 256, wsrs[h], ks * 512 + h * ws_half);
     };
     auto load_wtiles = [&](auto U, int kt) __attribute__((always_inline)) {
         constexpr int u = decltype(U)::value;
 #pragma unroll
         for(int j = 0; j < 4; j++)
-            vm_load_b128<0>(wf[u][j], w_voff[j & 1] + (j >> 1) * w_half, wrs[j >> 1], kt * 1024);
+            vm_load_b128<0>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
     };
 
-    // accumulator of (weight row group j, row group mt): acc[j][mt], or a[(j*MT + mt)*4 .. +3] when ACC_FIXED
-    v4f acc[4][ACC_FIXED ? 1 : MT];
+    // accumulator of (weight row group j, row group mt): a[(j*MT + mt)*4 .. +3]
     auto zero_acc = [&]() __attribute__((always_inline)) {
-        if constexpr(ACC_FIXED)
-            static_for<16 * MT>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
-        else
-        {
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-#pragma unroll
-                for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
-                    acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
-        }
+        static_for<16 * MT>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
     };
-    // the four accumulators of row group MTI (plus bias, when ACC_FIXED: there the bias is added here instead of
-    // being folded into the accumulators first)
-    auto fetch_row = [&](auto MTI, v4f (&row)[4], const float (&bz)[4][4]) __attribute__((always_inline)) {
+    // the four accumulators of row group MTI, plus bias (bias4(j) = the address of the lane's four bf16 biases of
+    // weight row group j; re-read per row group to keep the epilogue's register need small)
+    auto fetch_row = [&](auto MTI, v4f (&row)[4], auto bias4) __attribute__((always_inline)) {
         constexpr int mt = decltype(MTI)::value;
-        if constexpr(ACC_FIXED)
-        {
-            static_for<4>([&](auto J) __attribute__((always_inline)) {
-                constexpr int j = decltype(J)::value, a0 = (j * MT + mt) * 4;
-                row[j] = (v4f){acc_fixed_read<a0>() + bz[j][0], acc_fixed_read<a0 + 1>() + bz[j][1],
-                               acc_fixed_read<a0 + 2>() + bz[j][2], acc_fixed_read<a0 + 3>() + bz[j][3]};
-            });
-        }
-        else
-        {
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-                row[j] = acc[j][ACC_FIXED ? 0 : mt];
-        }
+        static_for<4>([&](auto J) __attribute__((always_inline)) {
+            constexpr int j = decltype(J)::value, a0 = (j * MT + mt) * 4;
+            row[j] = (v4f){acc_fixed_read<a0>(), acc_fixed_read<a0 + 1>(), acc_fixed_read<a0 + 2>(), acc_fixed_read<a0 + 3>()};
+            if(g.bias)
+            {
+                const uint2 b = *(const uint2*)bias4(j);
+                row[j][0] += bf16_bits_to_f32((uint16_t)b.x);
+                row[j][1] += bf16_bits_to_f32((uint16_t)(b.x >> 16));
+                row[j][2] += bf16_bits_to_f32((uint16_t)b.y);
+                row[j][3] += bf16_bits_to_f32((uint16_t)(b.y >> 16));
+            }
+        });
     };
 
     // ---------------------------------------------------------------- epilogue of one tile
-    auto epilogue = [&](const TileId& t, const u32* meta) __attribute__((always_inline)) {
+    auto epilogue = [&](const TileId& t, const u32* meta, int ma_t) __attribute__((always_inline)) {
         if(STAGE == 1)
         {
             // lane (r, kb) holds channels j*16 + kb*4 .. +3 (j = 0, 1) of row r.  After one permlane16 swap per
@@ -431,48 +435,36 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             typedef unsigned v2u __attribute__((ext_vector_type(2)));
             uint16_t* out = (uint16_t*)g.out;
             const int chw = t.nt * 128 + wave * 32;
-            float bz[4][4] = {};
-            if(g.bias)      // rare: fold the biases into the accumulators first
-            {
-#pragma unroll
-                for(int j = 0; j < 4; j++)
-                {
-#pragma unroll
-                    for(int i = 0; i < 4; i++)
-                        bz[j][i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4 + i]);
-                    if constexpr(!ACC_FIXED)
-                    {
-#pragma unroll
-                        for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
-#pragma unroll
-                            for(int i = 0; i < 4; i++)
-                                acc[j][mt][i] += bz[j][i];
-                    }
-                }
-            }
+            auto bz = [&](int j) __attribute__((always_inline)) {
+                return g.bias + (size_t)t.e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4;
+            };
             // after the swap: lane rows 0..3 hold channel offsets 0, 16, 8, 24
             const int ch_out = chw + (kb & 1) * 16 + (kb >> 1) * 8;
             static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
                 constexpr int mt = decltype(MTI)::value;
-                v4f row[4];
-                fetch_row(MTI, row, bz);
-                const int p   = t.m_blk * BM + mt * 16 + r;
-                const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
-                u32 d[2][2];
-#pragma unroll
-                for(int j = 0; j < 2; j++)
+                const int p = t.m_blk * BM + mt * 16 + r;
+                uint4 o     = make_uint4(0u, 0u, 0u, 0u);     // row groups that were skipped store zeros
+                if(mt < ma_t)
                 {
-                    float v[4];
+                    v4f row[4];
+                    fetch_row(MTI, row, bz);
+                    const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
+                    u32 d[2][2];
 #pragma unroll
-                    for(int i = 0; i < 4; i++)
-                        v[i] = ok ? silu_f32(row[j][i]) * row[j + 2][i] : 0.f;
-                    d[j][0] = pack_bf16x2(v[0], v[1]);
-                    d[j][1] = pack_bf16x2(v[2], v[3]);
+                    for(int j = 0; j < 2; j++)
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int i = 0; i < 4; i++)
+                            v[i] = ok ? silu_f32(row[j][i]) * row[j + 2][i] : 0.f;
+                        d[j][0] = pack_bf16x2(v[0], v[1]);
+                        d[j][1] = pack_bf16x2(v[2], v[3]);
+                    }
+                    v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
+                    v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
+                    // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
+                    o = make_uint4(t0.x, t1.x, t0.y, t1.y);
                 }
-                v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
-                v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
-                // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
-                const uint4 o = make_uint4(t0.x, t1.x, t0.y, t1.y);
                 if(out)
                     *(uint4*)(out + (size_t)p * I + ch_out) = o;
                 if(g.out_q)
@@ -502,27 +494,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             // four lane rows gives every lane 16 consecutive channels: 32 B stores, 128 B contiguous per row.
             uint16_t* out = (uint16_t*)g.out;
             const int chw = t.nt * 256 + wave * 64;
-            float bz[4][4] = {};
-            if(g.bias)      // rare: fold the bias into the accumulators first
-            {
-#pragma unroll
-                for(int j = 0; j < 4; j++)
-                {
-#pragma unroll
-                    for(int i = 0; i < 4; i++)
-                        bz[j][i] = bf16_bits_to_f32(g.bias[(size_t)t.e * g.N + chw + j * 16 + kb * 4 + i]);
-                    if constexpr(!ACC_FIXED)
-                    {
-#pragma unroll
-                        for(int mt = 0; mt < (ACC_FIXED ? 1 : MT); mt++)
-#pragma unroll
-                            for(int i = 0; i < 4; i++)
-                                acc[j][mt][i] += bz[j][i];
-                    }
-                }
-            }
+            auto bz = [&](int j) __attribute__((always_inline)) { return g.bias + (size_t)t.e * g.N + chw + j * 16 + kb * 4; };
             static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
                 constexpr int mt = decltype(MTI)::value;
+                if(mt >= ma_t)
+                    return;
                 v4f row[4];
                 fetch_row(MTI, row, bz);
                 const u32 id   = meta[mt * 16 + r];
@@ -557,6 +533,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         return;
     int mb = 0;                                   // meta buffer of the current tile (ring of 3)
     setup_load(cur, g.sorted_ids + (size_t)cur.m_blk * BM);
+    int ma     = count_groups(g.sorted_ids + (size_t)cur.m_blk * BM);   // active row groups of the current tile
+    int ma_nxt = ma;                                                    // ... and of the next one
     // prologue, in the K-group's issue order: this tile's ids/weights, activation K-group 0, weight scales of
     // group 0, weight tiles of K-steps 0..3
     dma_meta(cur, 0, true);
@@ -570,7 +548,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
 
     // one K-group; returns false when the workgroup has no more work
     auto kgroup = [&](auto P) __attribute__((always_inline)) -> bool {
-        constexpr int p = decltype(P)::value;     // parity of the global K-group count: LDS stage / scale registers
+        constexpr int p  = decltype(P)::value;    // parity of the global K-group count: LDS stage / scale registers
         const bool last     = ks == KS - 1;
         const int kpre      = last ? 0 : ks + 1;  // K-group that is prefetched now (of the next tile when last)
         const int mb_nxt    = mb == 2 ? 0 : mb + 1;
@@ -581,7 +559,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         if(last)
         {
             if(nxt.valid)
+            {
                 setup_load(nxt, lds_meta[mb_nxt]);
+                ma_nxt = count_groups(lds_meta[mb_nxt]);
+            }
             else
                 setup_null();
         }
@@ -615,19 +596,24 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             else
             {
                 constexpr int h = (k - NM - 5 * NA) / 2, c = (k - NM - 5 * NA) % 2;
-                vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256 + h * ws_half, wsrs[h], kpre * 512);
+                vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256, wsrs[h], kpre * 512 + h * ws_half);
             }
         };
+        // MFMAs, prefetches and weight loads of the K-group for a tile with MA active row groups (the prefetches
+        // always cover whole tiles).  One instance per MA; everything else in the K-group is shared.
+        auto body = [&](auto MAV) __attribute__((always_inline)) {
+        constexpr int MA  = decltype(MAV)::value;
+        constexpr int PPM = (NPF + MA - 1) / MA;  // prefetch operations issued after each row group's MFMAs
         constexpr int RA = 4;
         v4i af_r[RA + 1];
-        int asc_all[ACC_FIXED ? MT : 1];         // the scale dword of a row group serves all four K-steps
+        int asc_all[RING ? MT : 1];              // the scale dword of a row group serves all four K-steps
         auto lds_read = [&](auto NN) __attribute__((always_inline)) {
-            constexpr int n = decltype(NN)::value, uu = n / MT, mm = n % MT;
+            constexpr int n = decltype(NN)::value, uu = n / MA, mm = n % MA;
             af_r[n % (RA + 1)] = *(const v4i*)(stage[p] + (uu * SLOTS + mm) * 1024 + rd_a);
             if constexpr(uu == 0)
-                asc_all[ACC_FIXED ? mm : 0] = *(const int*)(sstage[p] + mm * 256 + rd_s);
+                asc_all[RING ? mm : 0] = *(const int*)(sstage[p] + mm * 256 + rd_s);
         };
-        if constexpr(ACC_FIXED)
+        if constexpr(RING)
             static_for<RA>([&](auto NN) __attribute__((always_inline)) { lds_read(NN); });
         __builtin_amdgcn_sched_barrier(0);
         static_for<4>([&](auto U) __attribute__((always_inline)) {
@@ -644,24 +630,24 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             // the one-wave-per-SIMD 256-row tile, where nothing else covers the LDS latency
             v4i af  = {0, 0, 0, 0};
             int asc = 0;
-            if constexpr(!ACC_FIXED)
+            if constexpr(!RING)
             {
                 af  = *(const v4i*)(stage[p] + (u * SLOTS) * 1024 + rd_a);
                 asc = *(const int*)(sstage[p] + rd_s);
             }
-            static_for<MT>([&](auto M) __attribute__((always_inline)) {
+            static_for<MA>([&](auto M) __attribute__((always_inline)) {
                 constexpr int mt = decltype(M)::value;
                 v4i af_n  = af;
                 int asc_n = asc;
-                if constexpr(ACC_FIXED)
+                if constexpr(RING)
                 {
-                    constexpr int n = u * MT + mt;             // position in the K-group's sequence of row groups
-                    if constexpr(n + RA < 4 * MT)
+                    constexpr int n = u * MA + mt;             // position in the K-group's sequence of row groups
+                    if constexpr(n + RA < 4 * MA)
                         lds_read(std::integral_constant<int, n + RA>{});
                     af  = af_r[n % (RA + 1)];
-                    asc = asc_all[ACC_FIXED ? mt : 0];
+                    asc = asc_all[RING ? mt : 0];
                 }
-                else if constexpr(mt + 1 < MT)
+                else if constexpr(mt + 1 < MA)
                 {
                     af_n  = *(const v4i*)(stage[p] + (u * SLOTS + mt + 1) * 1024 + rd_a);
                     asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
@@ -669,21 +655,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 __builtin_amdgcn_sched_barrier(0);
                 {
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                if constexpr(ACC_FIXED)
-                {
-                    mfma_fp4_fixed<(u & 1) * 2 + 0, u, (0 * MT + mt) * 4>(wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
-                    mfma_fp4_fixed<(u & 1) * 2 + 1, u, (1 * MT + mt) * 4>(wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
-                    mfma_fp4_fixed<(u & 1) * 2 + 0, u, (2 * MT + mt) * 4>(wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
-                    mfma_fp4_fixed<(u & 1) * 2 + 1, u, (3 * MT + mt) * 4>(wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
-                }
-                else
-                {
-                    constexpr int am = ACC_FIXED ? 0 : mt;
-                    mfma_fp4<(u & 1) * 2 + 0, u>(acc[0][am], wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
-                    mfma_fp4<(u & 1) * 2 + 1, u>(acc[1][am], wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
-                    mfma_fp4<(u & 1) * 2 + 0, u>(acc[2][am], wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
-                    mfma_fp4<(u & 1) * 2 + 1, u>(acc[3][am], wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
-                }
+                mfma_fp4_fixed<(u & 1) * 2 + 0, u, (0 * MT + mt) * 4>(wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
+                mfma_fp4_fixed<(u & 1) * 2 + 1, u, (1 * MT + mt) * 4>(wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
+                mfma_fp4_fixed<(u & 1) * 2 + 0, u, (2 * MT + mt) * 4>(wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
+                mfma_fp4_fixed<(u & 1) * 2 + 1, u, (3 * MT + mt) * 4>(wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
                 }
                 // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
                 // issue overlaps the matrix pipeline instead of preceding it
@@ -694,7 +669,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                             prefetch_op(std::integral_constant<int, k>{});
                     });
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr(!ACC_FIXED)
+                if constexpr(!RING)
                 {
                     af  = af_n;
                     asc = asc_n;
@@ -705,6 +680,19 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             load_wtiles(U, kpre * 4 + u);
             __builtin_amdgcn_sched_barrier(0);
         });
+        };
+        // largest count (the common case) tested first
+        {
+            bool done = false;
+            static_for<MT / MA_STEP>([&](auto V) __attribute__((always_inline)) {
+                constexpr int MA = MT - decltype(V)::value * MA_STEP;
+                if(!done && (MA == MA_STEP || ma == MA))
+                {
+                    body(std::integral_constant<int, MA>{});
+                    done = true;
+                }
+            });
+        }
         // (5) the 16 weight loads above are the only VMEM ops younger than this group's DMAs
         wait_vmcnt_barrier<16>();
         ks++;
@@ -713,10 +701,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             // the last MFMAs were issued from assembly: give their results the documented distance to the
             // first VALU read
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-            epilogue(cur, lds_meta[mb]);
+            epilogue(cur, lds_meta[mb], ma);
             if(!nxt.valid)
                 return false;
             cur = nxt;
+            ma  = ma_nxt;
             mb  = mb_nxt;
             ks  = 0;
             zero_acc();
@@ -772,7 +761,7 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
     PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256,
                   "%s: block_m=%d not in {16,32,64,128,256}", name, block_m);
     PYHIP_REQUIRE(n_blk >= 0 && n_blk < (1 << 24), "%s: n_blk=%lld", name, (long long)n_blk);
-    PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < (1ll << 32),
+    PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < 0xFFFF0000ll,
                   "%s: activation matrix of %lld rows x %d exceeds the 4 GiB buffer range", name, (long long)a_rows, K);
     PYHIP_REQUIRE(((uintptr_t)a_q % 16) == 0 && ((uintptr_t)a_s % 4) == 0 && ((uintptr_t)w % 16) == 0 &&
                       ((uintptr_t)w_s % 4) == 0 && ((uintptr_t)out % 8) == 0,
