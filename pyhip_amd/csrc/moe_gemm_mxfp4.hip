@@ -398,11 +398,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             for(int c = 0; c < 2; c++)
                 vm_load_b32<0>(w_sc[s][h * 2 + c], lane * 4 + c * 256, wsrs[h], ks * 512 + h * ws_half);
     };
+    auto load_wtile = [&](auto U, auto J, int kt) __attribute__((always_inline)) {
+        constexpr int u = decltype(U)::value, j = decltype(J)::value;
+        vm_load_b128<0>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
+    };
     auto load_wtiles = [&](auto U, int kt) __attribute__((always_inline)) {
-        constexpr int u = decltype(U)::value;
-#pragma unroll
-        for(int j = 0; j < 4; j++)
-            vm_load_b128<0>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
+        static_for<4>([&](auto J) __attribute__((always_inline)) { load_wtile(U, J, kt); });
     };
 
     // accumulator of (weight row group j, row group mt): a[(j*MT + mt)*4 .. +3]
@@ -621,7 +622,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             constexpr int u = decltype(U)::value;
             // (3) MFMAs of K-step 4*ks + u, tile operands two reads ahead of their MFMAs.  The weight tiles of
             //     this K-step (and, at u = 0, the weight scales) were requested one K-group ago.
-            constexpr int YOUNGER = u == 0 ? 12 : 12 + NPF;
+            //     Issue order of a K-group: the prefetches during K-step 0; the tiles of K-steps 0, 1, 2 of the
+            //     prefetched K-group one at a time during K-steps 1, 2, 3 (spread over the row groups: four 1 KB loads
+            //     back to back from every wave at once fill the address unit's queue and stall the issuing waves);
+            //     the tiles of K-step 3 after K-step 3.  Younger than the tiles of K-step u when it starts: u = 0: those
+            //     of K-steps 1, 2, 3; u = 1, 2, 3: two more K-steps' tiles and this K-group's prefetches.
+            constexpr int YOUNGER = u == 0 ? 12 : 8 + NPF;
             wait_vm_tiles<YOUNGER>(wf[u][0], wf[u][1], wf[u][2], wf[u][3]);
             if(u == 0)
                 wait_vm_scales<YOUNGER>(w_sc[p][0], w_sc[p][1], w_sc[p][2], w_sc[p][3]);
@@ -669,6 +675,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                         if constexpr(k < NPF)
                             prefetch_op(std::integral_constant<int, k>{});
                     });
+                // (4) weight tiles of the previous K-step of the prefetched K-group into the registers it consumed
+                if constexpr(u > 0)
+                    static_for<4>([&](auto J) __attribute__((always_inline)) {
+                        if constexpr(mt == (decltype(J)::value * MA) / 4)
+                            load_wtile(std::integral_constant<int, u - 1>{}, J, kpre * 4 + u - 1);
+                    });
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr(!RING)
                 {
@@ -677,8 +689,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
-            // (4) weight tiles of the same K-step of the prefetched K-group into the registers just consumed
-            load_wtiles(U, kpre * 4 + u);
+            if constexpr(u == 3)
+                load_wtiles(U, kpre * 4 + u);
             __builtin_amdgcn_sched_barrier(0);
         });
         };
