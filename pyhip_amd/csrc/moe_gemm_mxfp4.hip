@@ -121,6 +121,14 @@ __device__ __forceinline__ void vm_dma_b32(int voff, v4i rsrc, int soff, u32 lds
     asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen offset:%4 lds"
                  ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
 }
+// The same for descriptors that were just made uniform with v_readfirstlane: a vector-memory instruction must not
+// read a scalar register earlier than 5 wait states after a vector instruction wrote it, and the compiler does
+// not look into inline assembly for that (tests/test_build_checks.py scans the generated code for the pattern).
+__device__ __forceinline__ void vm_dma_b32_fresh_sgprs(int voff, v4i rsrc, u32 lds_base)
+{
+    asm volatile("s_nop 4\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
+                 ::"v"(voff), "s"(rsrc), "s"(lds_base) : "memory");
+}
 __device__ __forceinline__ u32 lds_addr_of(const void* p)
 {
     return (u32)(unsigned long long)(__attribute__((address_space(3))) const void*)p;
@@ -288,7 +296,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
             const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
             const u32 dst   = uni(real ? lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
-            vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
+            vm_dma_b32_fresh_sgprs((oo * 64 + lane) * 4, rs, dst);
         }
     };
 
@@ -315,17 +323,19 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         asrs = make_rsrc(g.a_s, 0);
     };
     // Row groups of a tile that hold at least one real row.  The sort pads every expert's rows at the END of
-    // its last block, so the real rows of a block are a prefix: padded row groups are skipped by the MFMA loop
-    // (kgroup<.., MA>) and their activation fetches are sent out of the descriptor's range, where the
-    // hardware drops them.  Rounded up to the granularity the K-group body is instantiated for.
-    constexpr int MA_STEP = MT > 8 ? 2 : MT;
-    constexpr u32 OOB     = 0xFFFF0000u;           // beyond every activation buffer (checked by the launcher)
+    // its last block, so the real rows of a block are a prefix.  Padded rows send their activation fetches out
+    // of the descriptor's range, where the hardware drops them, and the epilogue leaves padded row groups out.
+    // Their MFMAs are still issued: the K-group body exists once.  (Instantiating it per count of active row
+    // groups and branching between the instances is NOT safe with this pipeline: the register allocator then
+    // gives the weight-tile registers different homes in different instances and copies them at the joins,
+    // while loads into them are still in flight, which it cannot know.  Measured: wrong results in tiles that
+    // run short K-groups.  tests/test_build_checks.py looks for such copies in the generated code.)
+    constexpr u32 OOB = 0xFFFF0000u;               // beyond every activation buffer (checked by the launcher)
     auto count_groups = [&](const u32* ids) __attribute__((always_inline)) -> int {
         const u32 id  = ids[(lane < MT ? lane : 0) * 16];
         const bool ok = lane < MT && (int)(id >> 24) < g.topk && (int)(id & 0xFFFFFFu) < g.T;
-        int n         = __builtin_popcountll(__ballot(ok));
-        n             = n < 1 ? 1 : n;
-        return (n + MA_STEP - 1) / MA_STEP * MA_STEP;
+        const int n   = __builtin_popcountll(__ballot(ok));
+        return n < 1 ? 1 : n;
     };
     // ids: the tile's sorted ids, either in LDS (meta buffer) or in global memory
     auto setup_load = [&](const TileId& t, const u32* ids) __attribute__((always_inline)) {
@@ -585,7 +595,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
                 const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
                 const u32 dst   = uni(real ? lds_addr_of(&lds_meta[mb_nxt][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
-                vm_dma_b32<0, 0>((oo * 64 + lane) * 4, rs, 0, dst);
+                vm_dma_b32_fresh_sgprs((oo * 64 + lane) * 4, rs, dst);
             }
             else if constexpr(k < NM + 5 * NA)
             {
@@ -601,10 +611,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256, wsrs[h], kpre * 512 + h * ws_half);
             }
         };
-        // MFMAs, prefetches and weight loads of the K-group for a tile with MA active row groups (the prefetches
-        // always cover whole tiles).  One instance per MA; everything else in the K-group is shared.
-        auto body = [&](auto MAV) __attribute__((always_inline)) {
-        constexpr int MA  = decltype(MAV)::value;
+        // MFMAs, prefetches and weight loads of the K-group
+        constexpr int MA  = MT;                   // row groups that take part
         constexpr int PPM = (NPF + MA - 1) / MA;  // prefetch operations issued after each row group's MFMAs
         constexpr int RA = 4;
         v4i af_r[RA + 1];
@@ -693,19 +701,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 load_wtiles(U, kpre * 4 + u);
             __builtin_amdgcn_sched_barrier(0);
         });
-        };
-        // largest count (the common case) tested first
-        {
-            bool done = false;
-            static_for<MT / MA_STEP>([&](auto V) __attribute__((always_inline)) {
-                constexpr int MA = MT - decltype(V)::value * MA_STEP;
-                if(!done && (MA == MA_STEP || ma == MA))
-                {
-                    body(std::integral_constant<int, MA>{});
-                    done = true;
-                }
-            });
-        }
         // (5) the 16 weight loads above are the only VMEM ops younger than this group's DMAs
         wait_vmcnt_barrier<16>();
         ks++;

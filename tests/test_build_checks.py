@@ -41,3 +41,97 @@ def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(tmp_path):
         assert hand["mfma"] and hand["read"] and hand["write"], (name, hand)
         m = re.search(r"ScratchSize: (\d+)", text[text.index(name):])
         assert m and int(m.group(1)) == 0, (name, "spills")
+
+
+def _instructions(body):
+    for line in body.split("\n"):
+        code = line.split(";")[0].strip()
+        if code and not code.startswith(".") and not code.endswith(":"):
+            yield code
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
+def test_no_vector_written_scalar_register_is_read_too_early_by_vector_memory(tmp_path):
+    """gfx9 hazard: a vector-memory instruction may read a scalar register only 5 wait states after a vector
+    instruction (v_readlane / v_readfirstlane) wrote it.  The compiler pads its own instructions but not the
+    hand-written ones inside inline assembly, so the generated code of every GEMM kernel is scanned."""
+    from pyhip_amd import build
+    out = tmp_path / "gemm.s"
+    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
+    assert len(kernels) == 10
+    for name, body in kernels:
+        ins = list(_instructions(body))
+        for i, line in enumerate(ins):
+            m = re.match(r"v_(?:readlane|readfirstlane)_b32 s(\d+),", line)
+            if not m:
+                continue
+            sreg, waited = int(m.group(1)), 0
+            for nxt in ins[i + 1:i + 8]:
+                if re.match(r"(buffer_|global_|scratch_|flat_)", nxt):
+                    used = set()
+                    for a, b in re.findall(r"s\[(\d+):(\d+)\]", nxt):
+                        used.update(range(int(a), int(b) + 1))
+                    used.update(int(a) for a in re.findall(r"\bs(\d+)\b", nxt))
+                    assert sreg not in used or waited >= 5, (name, line, nxt, waited)
+                nop = re.match(r"s_nop (\d+)", nxt)
+                waited += int(nop.group(1)) + 1 if nop else 1
+                if waited >= 5:
+                    break
+
+
+def _vgprs(operand_text):
+    regs = set()
+    for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", operand_text):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(a) for a in re.findall(r"\bv(\d+)\b", operand_text))
+    return regs
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
+def test_compiler_never_copies_a_register_with_a_load_in_flight(tmp_path):
+    """The weight tiles and weight scales are loaded by inline assembly long before they are used, and only the
+    hand-written waits know when they have arrived.  That holds as long as the compiler leaves those registers
+    alone: a copy it inserts (live-range splitting, a join between two instances of a loop body) would read a
+    register whose load is still in flight.  Check: outside the inline-assembly regions no instruction of a GEMM
+    kernel reads or writes a register that an inline-assembly load writes to."""
+    from pyhip_amd import build
+    out = tmp_path / "gemm.s"
+    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
+    assert len(kernels) == 10
+    for name, body in kernels:
+        # Walk the kernel text: a register is "loaded" from the inline-assembly load that writes it until the
+        # compiler's own code overwrites it with something else.  Values loaded that way are consumed by
+        # inline-assembly MFMAs only, so no instruction of the compiler may READ a register in that state.
+        inside, loaded, seen = False, set(), set()
+        for line in body.split("\n"):
+            if "ASMSTART" in line:
+                inside = True
+            elif "ASMEND" in line:
+                inside = False
+            else:
+                code = line.split(";")[0].strip()
+                if not code or code.startswith(".") or code.endswith(":"):
+                    continue
+                if inside:
+                    m = re.match(r"buffer_load_dword(?:x4)? (v\[\d+:\d+\]|v\d+), (?!.*\blds\b)", code)
+                    if m:
+                        loaded |= _vgprs(m.group(1))
+                        seen |= _vgprs(m.group(1))
+                    m = re.match(r"v_accvgpr_read_b32 (v\d+),", code)      # epilogue: a new value for that register
+                    if m:
+                        loaded -= _vgprs(m.group(1))
+                elif code.startswith(("v_", "ds_", "buffer_", "global_", "scratch_", "flat_")):
+                    mnemonic, _, operands = code.partition(" ")
+                    ops = operands.split(",")
+                    stores = "store" in mnemonic or "write" in mnemonic or mnemonic.startswith("v_cmp")
+                    written = set() if stores else _vgprs(ops[0])
+                    read = _vgprs(operands if stores else ",".join(ops[1:]))
+                    assert not (read & loaded), (name, code, sorted(read & loaded))
+                    loaded -= written
+        assert len(seen) >= 64 + 8, (name, len(seen))        # 16 weight tiles of 4 registers, 8 scale dwords

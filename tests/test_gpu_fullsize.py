@@ -89,3 +89,20 @@ def test_sampled_experts_and_properties(layer, T, method):
     rev = torch.arange(k - 1, -1, -1, device="cuda")
     _, parts_r = _run(W, hidden, tw[:, rev].contiguous(), ti[:, rev].contiguous(), return_parts=True, method=method)
     assert torch.equal(parts_r["out3"][:, rev], out3)
+
+
+def test_tile_heights_agree_bit_for_bit(layer):
+    """128-row and 256-row tiles compute every routed row with the same instructions in the same order, so the
+    layer output must not depend on block_size_M.  At T=8192 about half of the experts have a few rows more than
+    256: their second 256-row block is almost empty, its K-groups are short, and every hand-counted wait of the
+    pipeline really has to hold (a data race in the 256-row tile showed up exactly there)."""
+    W = layer
+    T = 8192
+    from pyhip_amd import workloads
+    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
+    print(f"full-size case {SHAPE} T={T} block_size_M 64 / 128 / 256", flush=True)
+    outs = {bm: _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm) for bm in (64, 128, 256)}
+    torch.cuda.synchronize()
+    assert torch.isfinite(outs[128].float()).all()
+    assert torch.equal(outs[64], outs[128])
+    assert torch.equal(outs[256], outs[128])
