@@ -87,8 +87,10 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
                               uint8_t* scales, const uint32_t* rows_limit, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
- * Stage 1: gate_up grouped GEMM with fused SiLU(gate)*up.  Replaces moe_gemm_mxfp4(gate_up=True),
+ * Stage 1: gate_up grouped GEMM with the fused gated activation.  Replaces moe_gemm_mxfp4(gate_up=True),
  * src/contrib/moe_gemm_mxfp4.py:972-1290 (launch: tests/contrib/moe/test_moe.py:720-730).
+ *   activation   0: SiLU(gate) * up;  1: gpt-oss's clamped SwiGLU, min(gate, L) * sigmoid(1.702 * min(gate, L)) *
+ *                (clamp(up, -L, L) + 1) with L = swiglu_limit > 0 (tests/contrib/moe/test_moe.py:73-82)
  *   a_q/a_scale  quantised hidden states [tokens, hidden/2] / scales (token order, see above)
  *   w1           u8 [experts, 2*inter, hidden/2], gate rows then up rows, pre-shuffled as
  *                src/misc.py:116-130 (pre_shuffle(x, 16))
@@ -107,7 +109,7 @@ int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
                           const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q,
                           uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                          int64_t n_blk, pyhip_stream_t stream);
+                          int64_t n_blk, int activation, float swiglu_limit, pyhip_stream_t stream);
 
 /* Stage 2: down grouped GEMM, times the routing weight.  Replaces moe_gemm_mxfp4(gate_up=False),
  * src/contrib/moe_gemm_mxfp4.py:1291-1333 (launch: tests/contrib/moe/test_moe.py:751-763).
@@ -132,11 +134,12 @@ int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const ui
  * adding into the layer output with atomics.  block_m is 16, 32 or 64; hidden % 512 == 0, inter % 512 == 0.
  * split_k: 4 = the four waves of a workgroup share a 64-row weight tile and split K between them (partial sums
  * meet in LDS; four times as many workgroups), 1 = every wave owns 64 rows over the whole K, 0 = split when the
- * launch would otherwise have fewer than 2048 workgroups with work. */
+ * launch would otherwise have fewer than 2048 workgroups with work.  activation / swiglu_limit: as for
+ * pyhip_moe_gemm1_mxfp4. */
 int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale, const void* bias1_bf16,
                           const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
                           void* a2_bf16, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                          int64_t n_blk, int split_k, pyhip_stream_t stream);
+                          int64_t n_blk, int split_k, int activation, float swiglu_limit, pyhip_stream_t stream);
 int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale, const void* bias2_bf16,
                           const uint32_t* sorted_ids, const float* sorted_weights, const uint32_t* sorted_expert_ids,
                           const uint32_t* num_valid_ids, void* out3_bf16, int tokens, int topk, int experts,

@@ -45,12 +45,24 @@ def expert_weights_f32(wq, ws):
     return mxfp4.dequantize_mxfp4(wq, ws)
 
 
-def gateup_ref(x, w1, bias1=None):
-    """x f32 [n, H], w1 f32 [2I, H] -> bf16-rounded silu(gate) * up, f32 [n, I]"""
+def swiglu(gate, up, limit=None):
+    """gpt-oss's gated activation as the reference states it (tests/contrib/moe/test_moe.py:76-81): the gate is
+    clamped from above only, the up projection from both sides, limit 7.0 when none is given."""
+    limit = float(limit) if limit else 7.0
+    g = _t(np.asarray(gate, dtype=np.float32)).clamp(max=limit)
+    u = _t(np.asarray(up, dtype=np.float32)).clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).numpy()
+
+
+def gateup_ref(x, w1, bias1=None, activation="silu", swiglu_limit=None):
+    """x f32 [n, H], w1 f32 [2I, H] -> bf16-rounded silu(gate) * up (or swiglu(gate, up)), f32 [n, I]"""
     acc = torch.matmul(_t(x), _t(w1).t()).numpy()
     if bias1 is not None:
         acc = acc + np.asarray(bias1, dtype=np.float32)[None, :]
     I = w1.shape[0] // 2
+    if activation == "swiglu":
+        return mxfp4.bf16_round(swiglu(acc[:, :I], acc[:, I:], swiglu_limit))
+    assert activation == "silu"
     return mxfp4.bf16_round(silu(acc[:, :I]) * acc[:, I:])
 
 
@@ -63,7 +75,7 @@ def down_ref(a2, w2, weight, bias2=None):
 
 
 def moe_ref(hidden, w1q, w1s, w2q, w2s, topk_weight, topk_ids, *, act="a4",
-            bias1=None, bias2=None, experts=None, return_parts=False):
+            bias1=None, bias2=None, experts=None, return_parts=False, activation="silu", swiglu_limit=None):
     """Whole layer.
 
     hidden      float32 [T, H] holding bf16 values
@@ -89,7 +101,7 @@ def moe_ref(hidden, w1q, w1s, w2q, w2s, topk_weight, topk_ids, *, act="a4",
             continue
         w1 = expert_weights_f32(w1q[e], w1s[e])
         w2 = expert_weights_f32(w2q[e], w2s[e])
-        a2 = gateup_ref(x_in[tok], w1, None if bias1 is None else bias1[e])
+        a2 = gateup_ref(x_in[tok], w1, None if bias1 is None else bias1[e], activation, swiglu_limit)
         a2_all[tok, slot] = a2
         a2_in = act_quant_dequant(a2) if act == "a4" else a2
         per_slot[tok, slot] = down_ref(a2_in, w2, topk_weight[tok, slot],

@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpyhip_moe.so")
 
 _c = ctypes
-_P, _I, _L = _c.c_void_p, _c.c_int, _c.c_int64
+_P, _I, _L, _F = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
 
 #: symbol -> (restype, argtypes); the single source the loader and the export test share
 SIGNATURES = {
@@ -23,9 +23,9 @@ SIGNATURES = {
     "pyhip_moe_sorting": (_I, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _P]),
     "pyhip_moe_act_scale_stride": (_L, [_I]),
     "pyhip_moe_act_quant_mxfp4": (_I, [_P, _L, _L, _I, _P, _P, _P, _P]),
-    "pyhip_moe_gemm1_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
+    "pyhip_moe_gemm1_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _F, _P]),
     "pyhip_moe_gemm2_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
-    "pyhip_moe_gemm1_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _P]),
+    "pyhip_moe_gemm1_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _P]),
     "pyhip_moe_gemm2_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _P]),
     "pyhip_moe_topk_reduce": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),
 }

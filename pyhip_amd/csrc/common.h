@@ -56,6 +56,43 @@ __device__ __forceinline__ float silu_f32(float x)
     return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// gpt-oss's gated activation (tests/contrib/moe/test_moe.py:76-81): the gate is clamped from above, the up
+// projection from both sides, out = gate * sigmoid(1.702 * gate) * (up + 1); same hardware approximations
+__device__ __forceinline__ float swiglu_f32(float gate, float up, float limit)
+{
+    gate    = fminf(gate, limit);
+    up      = fminf(fmaxf(up, -limit), limit);
+    float e = __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * gate);
+    return gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + 1.0f);
+}
+
+// The gated activation of the gate_up GEMMs in one branch-free form,
+//     g' * sigmoid(alpha * g') * (u' + beta),   g' = min(gate, limit),  u' = clamp(up, -limit, limit):
+// SiLU(gate) * up is alpha = 1, beta = 0, limit = +inf (the clamps then change nothing); gpt-oss's clamped SwiGLU
+// (tests/contrib/moe/test_moe.py:76-81) is alpha = 1.702, beta = 1 and its limit.  Same hardware approximations
+// as silu_f32.  Used by the bf16-activation GEMM; the MXFP4 GEMM is instantiated per activation instead (the extra
+// four instructions per element showed in its time, and a branch between two forms in its epilogue costs registers
+// the 128-row tile does not have).
+struct GatedAct
+{
+    float neg_alpha_log2e, beta, limit;
+};
+__device__ __host__ __forceinline__ GatedAct make_gated_act(int activation, float swiglu_limit)
+{
+    GatedAct a;
+    a.neg_alpha_log2e = -1.4426950408889634f * (activation ? 1.702f : 1.0f);
+    a.beta            = activation ? 1.0f : 0.0f;
+    a.limit           = activation ? swiglu_limit : __builtin_inff();
+    return a;
+}
+__device__ __forceinline__ float gated_act_f32(const GatedAct& a, float gate, float up)
+{
+    gate    = fminf(gate, a.limit);
+    up      = fminf(fmaxf(up, -a.limit), a.limit);
+    float e = __builtin_amdgcn_exp2f(a.neg_alpha_log2e * gate);
+    return gate * __builtin_amdgcn_rcpf(1.0f + e) * (up + a.beta);
+}
+
 // ---- MXFP4 quantisation of bf16 values (shared by the quantisation kernel and the stage-1 GEMM epilogue)
 // running maximum of the magnitudes (15-bit patterns) of the two bf16 halves of w
 __device__ __forceinline__ u32 amax15(u32 acc, u32 w)

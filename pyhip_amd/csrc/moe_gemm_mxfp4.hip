@@ -41,6 +41,7 @@ struct GemmArgs
     uint8_t* out_q;            // stage 1: MXFP4 of the output, e2m1 pairs [n_blk*BM, N/4], or null
     uint8_t* out_s;            //          and its scales [n_blk*BM, OSK] in the activation-scale layout
     int OSK;
+    float limit;               // stage 1, SwiGLU: the clamp
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
 };
 
@@ -182,7 +183,7 @@ struct TileId
 // the memory pipeline never drains between tiles.  One barrier per K-group (512 K elements).  Everything
 // a tile boundary needs (schedule tables, sorted ids, routing weights) is read from LDS, so no wait on the
 // vector-memory counter ever covers the prefetches in flight.
-template <int STAGE, int MT>
+template <int STAGE, int MT, int ACT>
 __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
@@ -468,7 +469,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                         float v[4];
 #pragma unroll
                         for(int i = 0; i < 4; i++)
-                            v[i] = ok ? silu_f32(row[j][i]) * row[j + 2][i] : 0.f;
+                            v[i] = !ok ? 0.f : ACT == 0 ? silu_f32(row[j][i]) * row[j + 2][i] : swiglu_f32(row[j][i], row[j + 2][i], g.limit);
                         d[j][0] = pack_bf16x2(v[0], v[1]);
                         d[j][1] = pack_bf16x2(v[2], v[3]);
                     }
@@ -732,7 +733,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
 }
 
 template <int STAGE>
-static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
+static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
 {
     unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
     if(g.K < 1024)
@@ -747,15 +748,20 @@ static int launch_gemm(GemmArgs g, int block_m, hipStream_t stream)
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
     dim3 grid(nwg), block(GEMM_THREADS);
+    // ACT (0 SiLU * up, 1 clamped SwiGLU) only exists for the gate_up stage
+#define GEMM_CASE(BM, MTV)                                                                                         \
+    case BM:                                                                                                       \
+        if(STAGE == 1 && act == 1)                                                                                 \
+            hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, STAGE == 1 ? 1 : 0>), grid, block, 0, stream, g); \
+        else                                                                                                       \
+            hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, 0>), grid, block, 0, stream, g);                  \
+        break;
     switch(block_m)
     {
-    case 16: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 1>), grid, block, 0, stream, g); break;
-    case 32: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 2>), grid, block, 0, stream, g); break;
-    case 64: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 4>), grid, block, 0, stream, g); break;
-    case 128: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 8>), grid, block, 0, stream, g); break;
-    case 256: hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, 16>), grid, block, 0, stream, g); break;
+        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(256, 16)
     default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256}", block_m); return PYHIP_ERR_INVALID;
     }
+#undef GEMM_CASE
     PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel");
     return PYHIP_OK;
 }
@@ -782,9 +788,11 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
                                      const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q, uint8_t* a2_scale,
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, hipStream_t stream)
+                                     int64_t n_blk, int activation, float swiglu_limit, hipStream_t stream)
 {
     PYHIP_REQUIRE(a2_bf16 || a2_q, "moe_gemm1: no output buffer");
+    PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
+                  "moe_gemm1: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
     PYHIP_REQUIRE((a2_q == nullptr) == (a2_scale == nullptr), "moe_gemm1: a2_q and a2_scale go together");
     PYHIP_REQUIRE(!a2_q || inter % 512 == 0, "moe_gemm1: quantised output needs inter=%d to be a multiple of 512", inter);
     PYHIP_REQUIRE(((uintptr_t)a2_q % 4) == 0 && ((uintptr_t)a2_bf16 % 16) == 0, "moe_gemm1: unaligned output");
@@ -800,12 +808,13 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
     g.a_q = a_q; g.a_s = a_scale; g.w = w1; g.w_s = w1_scale; g.bias = (const uint16_t*)bias1_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
     g.out = a2_bf16; g.out_q = a2_q; g.out_s = a2_scale; g.OSK = (inter + 511) / 512 * 16;
+    g.limit = swiglu_limit;
     g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
     g.SK = (hidden + 511) / 512 * 16;
     g.SC = (hidden / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = inter / 128; g.a_rows = tokens;
-    return launch_gemm<1>(g, block_m, stream);
+    return launch_gemm<1>(g, block_m, activation, stream);
 }
 
 extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2,
@@ -828,10 +837,11 @@ extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scal
     g.a_q = a2_q; g.a_s = a2_scale; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
     g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
     g.num_valid = num_valid_ids; g.out = out3_bf16; g.out_q = nullptr; g.out_s = nullptr; g.OSK = 0;
+    g.limit = 0.f;
     g.sched = schedule; g.E = experts;
     g.T = tokens; g.topk = topk; g.K = inter; g.N = hidden;
     g.SK = (inter + 511) / 512 * 16;
     g.SC = (inter / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
-    return launch_gemm<2>(g, block_m, stream);
+    return launch_gemm<2>(g, block_m, 0, stream);
 }

@@ -32,6 +32,7 @@ struct W4A16Args
     const u32* num_valid;      // [2]
     uint16_t* out;             // stage 1: bf16 [n_blk*BM, N/2]; stage 2: bf16 [T, topk, N]
     int T, topk, K, N, SC, n_tiles;
+    GatedAct act;              // stage 1: the gated activation (common.h)
 };
 
 // 32 e2m1 values (4 dwords) times 2^(scale byte - 127) -> four MFMA operands of 8 bf16
@@ -211,7 +212,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
                 float v[4];
 #pragma unroll
                 for(int i = 0; i < 4; i++)
-                    v[i] = ok[mt] ? silu_f32(acc[j][mt][i]) * acc[j + 2][mt][i] : 0.f;
+                    v[i] = ok[mt] ? gated_act_f32(g.act, acc[j][mt][i], acc[j + 2][mt][i]) : 0.f;
                 uint2 o = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
                 *(uint2*)(g.out + (size_t)p * I + chbase + j * 16 + kb * 4) = o;
             }
@@ -279,9 +280,12 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
                                      const void* bias1_bf16, const uint32_t* sorted_ids,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, void* a2_bf16,
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, int split_k, hipStream_t stream)
+                                     int64_t n_blk, int split_k, int activation, float swiglu_limit,
+                                     hipStream_t stream)
 {
     PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4, "moe_gemm1_w4a16: split_k=%d not in {0,1,4}", split_k);
+    PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
+                  "moe_gemm1_w4a16: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
     int rc = check_w4a16("moe_gemm1_w4a16", hidden_bf16, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                          a2_bf16, hidden, block_m, n_blk, inter / 128);
     if(rc)
@@ -295,6 +299,7 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
     g.sorted_ids = sorted_ids; g.sorted_w = nullptr; g.sorted_e = sorted_expert_ids; g.num_valid = num_valid_ids;
     g.out = (uint16_t*)a2_bf16; g.T = tokens; g.topk = topk; g.K = hidden; g.N = 2 * inter;
     g.SC = (hidden / 32 + 7) / 8 * 8; g.n_tiles = inter / 128;
+    g.act = make_gated_act(activation, swiglu_limit);
     return launch_w4a16<1>(g, block_m, n_blk, (int64_t)tokens * topk, experts, split_k, stream);
 }
 
@@ -319,5 +324,6 @@ extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, con
     g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
     g.num_valid = num_valid_ids; g.out = (uint16_t*)out3_bf16; g.T = tokens; g.topk = topk; g.K = inter;
     g.N = hidden; g.SC = (inter / 32 + 7) / 8 * 8; g.n_tiles = hidden / 256;
+    g.act = make_gated_act(0, 0.f);
     return launch_w4a16<2>(g, block_m, n_blk, (int64_t)tokens * topk, experts, split_k, stream);
 }

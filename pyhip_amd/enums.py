@@ -7,6 +7,7 @@ class ActivationType(enum.IntEnum):
     No = -1
     Silu = 0
     Gelu = 1
+    Swiglu = 2
 
 
 class QuantType(enum.IntEnum):

@@ -78,12 +78,17 @@ def fused_moe(
     method="auto",
     return_parts=False,
     stage_events=None,
+    swiglu_limit=None,
 ):
     """See the module docstring.  Extras beyond the reference signature: ``dtype=torch.float32`` returns
     the fp32 top-k sum without the final bf16 rounding; ``return_parts=True`` also returns the
-    intermediate buffers; ``stage_events`` (a list) receives ``(name, start_event, end_event)`` per stage."""
+    intermediate buffers; ``stage_events`` (a list) receives ``(name, start_event, end_event)`` per stage;
+    ``activation=ActivationType.Swiglu`` selects gpt-oss's clamped SwiGLU with ``swiglu_limit`` (default 7.0, as
+    tests/contrib/moe/test_moe.py:76-81)."""
     lib = _lib.load()
-    assert activation == ActivationType.Silu, "only SiLU-gated experts are implemented"
+    assert activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts"
+    act = 1 if activation == ActivationType.Swiglu else 0
+    limit = float(swiglu_limit) if swiglu_limit else 7.0
     assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
     assert not doweight_stage1
     assert a1_scale is None and a2_scale is None, "activations are quantised dynamically"
@@ -151,7 +156,7 @@ def fused_moe(
         a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
         rc = lib.pyhip_moe_gemm1_w4a16(_lib.dptr(hs), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(bias1),
                                        _lib.dptr(sorted_ids), _lib.dptr(sorted_e), _lib.dptr(num_valid),
-                                       _lib.dptr(a2), T, k, global_E, H, I, bm, n_blk, splitk, stream)
+                                       _lib.dptr(a2), T, k, global_E, H, I, bm, n_blk, splitk, act, limit, stream)
         _lib.check(rc, "moe_gemm1_w4a16")
         ev = _mark("gemm1", ev)
         out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
@@ -183,7 +188,7 @@ def fused_moe(
     rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                    _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
                                    _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
-                                   _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, stream)
+                                   _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, act, limit, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
     out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)

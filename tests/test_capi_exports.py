@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.pyhip_moe_abi_version() == 2
+    assert lib.pyhip_moe_abi_version() == 3
 
 
 def test_size_helpers():
@@ -46,7 +46,7 @@ def test_argument_errors_are_reported():
     one = ctypes.c_void_p(16)
     rc = lib.pyhip_moe_act_quant_mxfp4(one, 40, 4, 40, one, one, None, None)
     assert rc == 1 and b"multiple of 32" in lib.pyhip_moe_last_error()
-    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1000, 512, 16, 4, None)
+    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1000, 512, 16, 4, 0, 0.0, None)
     assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
     rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 48, 4, None)
     assert rc == 1 and b"block_m" in lib.pyhip_moe_last_error()

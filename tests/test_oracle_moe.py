@@ -99,3 +99,35 @@ def test_metrics_closed_forms():
     assert abs(metrics.calc_diff(x, 3 * x) - (1 - 6 / 10)) < 1e-12      # 1 - 2c/(1+c^2)
     assert abs(metrics.cosine(x, 5 * x) - 1) < 1e-12
     assert abs(metrics.max_err_over_rms(x + 0.5, x) - 0.5 / np.sqrt(np.mean(x.astype(np.float64) ** 2))) < 1e-12
+
+
+def test_swiglu_pins():
+    """gpt-oss's gated activation (tests/contrib/moe/test_moe.py:76-81) against the formula in float64 and against
+    the cases that tell its clamps apart: the gate is clamped from above ONLY, the up projection from both sides,
+    the limit defaults to 7."""
+    rng = np.random.default_rng(5)
+    g = rng.uniform(-6, 6, 1000).astype(np.float32)
+    u = rng.uniform(-6, 6, 1000).astype(np.float32)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    np.testing.assert_allclose(moe.swiglu(g, u), g64 / (1 + np.exp(-1.702 * g64)) * (u64 + 1), rtol=2e-6, atol=1e-6)
+
+    def closed(gv, uv):
+        return gv / (1 + np.exp(-1.702 * gv)) * (uv + 1)
+    one = np.ones(1, np.float32)
+    np.testing.assert_allclose(moe.swiglu(100 * one, 2 * one), closed(7.0, 2.0), rtol=1e-6)            # gate clamped above
+    assert abs(float(moe.swiglu(-100 * one, 2 * one)[0])) < 1e-30                                      # ... not below
+    assert abs(closed(-7.0, 2.0)) > 1e-5                                                               # (a symmetric clamp would show)
+    np.testing.assert_allclose(moe.swiglu(one, 100 * one), closed(1.0, 7.0), rtol=1e-6)                # up clamped above
+    np.testing.assert_allclose(moe.swiglu(one, -100 * one), closed(1.0, -7.0), rtol=1e-6)              # ... and below
+    np.testing.assert_allclose(moe.swiglu(3 * one, 3 * one, 0.5), closed(0.5, 0.5), rtol=1e-6)         # explicit limit
+    np.testing.assert_allclose(moe.swiglu(3 * one, 3 * one, None), moe.swiglu(3 * one, 3 * one, 7.0))  # default 7
+    assert float(moe.swiglu(0 * one, 0 * one)[0]) == 0.0                                               # zero padding stays zero
+    # through the gate_up restatement: identity-like weights, gate = 4x, up = 2x
+    H = I = 32
+    eye = np.eye(H, dtype=np.float32)
+    w1 = np.concatenate([4 * eye, 2 * eye])
+    x = mxfp4.bf16_round(np.linspace(-3, 3, 2 * H, dtype=np.float32).reshape(2, H))
+    got = moe.gateup_ref(x, w1, activation="swiglu", swiglu_limit=5.0)
+    gv, uv = np.minimum(4 * x.astype(np.float64), 5.0), np.clip(2 * x.astype(np.float64), -5.0, 5.0)
+    np.testing.assert_allclose(got, mxfp4.bf16_round(closed(gv, uv).astype(np.float32)), rtol=2 ** -7, atol=1e-6)
+    assert np.abs(got - moe.gateup_ref(x, w1)).max() > 0.1                                             # differs from SiLU
