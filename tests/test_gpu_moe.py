@@ -290,6 +290,29 @@ def test_swiglu_matches_oracle(method, limit, T):
     assert metrics.cosine(got, silu_ref) < 0.99                                 # and it is not SiLU
 
 
+def test_prepared_weight_file_feeds_the_operator(tmp_path):
+    """pyhip_amd.prepare_weights: float weights -> file -> operator arguments; same bytes and same output as the
+    weights the other tests build by hand (padded gpt-oss-like shape with biases)."""
+    from pyhip_amd import prepare_weights as pw
+    L = cases.make_layer("gptoss_s", 20, seed=6, bias=True)
+    w1f = torch.from_numpy(om.dequantize_mxfp4(L.w1q, L.w1s))          # exactly representable: quantising again is the identity
+    w2f = torch.from_numpy(om.dequantize_mxfp4(L.w2q, L.w2s))
+    path = str(tmp_path / "layer.safetensors")
+    pw.save(path, *pw.convert(w1f, w2f, L.bias1, L.bias2))
+    tensors, meta = pw.load(path, device="cuda")
+    (w1, w2), kw = pw.fused_moe_kwargs(tensors, meta)
+    r1, r1s, r2, r2s, b1, b2, hp, ip = cases.padded_device_weights(L)
+    assert (hp, ip) == (meta["hidden_pad"], meta["intermediate_pad"])
+    assert torch.equal(w1, r1) and torch.equal(w2, r2) and torch.equal(kw["w1_scale"], r1s) and torch.equal(kw["w2_scale"], r2s)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    print("prepared-weights case gptoss_s T=20", flush=True)
+    out = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, **kw)
+    ref = fused_moe(L.hidden.cuda(), r1, r2, tw, ti, w1_scale=r1s, w2_scale=r2s, bias1=b1, bias2=b2, hidden_pad=hp,
+                    intermediate_pad=ip)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref) and torch.isfinite(out.float()).all()
+
+
 def test_auto_dispatch():
     """method="auto": bf16 activations up to 2 routed rows per expert on average, MXFP4 activations above"""
     L = cases.make_layer("dsv3_s", 16, seed=2)            # 16 * 8 / 64 = 2 rows per expert
