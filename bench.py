@@ -166,7 +166,10 @@ def main():
         "stage_ms": {k: round(v, 4) for k, v in main_res["stage_ms"].items()},
         "roofline": {"kernel": "moe_gemm_mxfp4_kernel<1,*> (gate_up)", "bound": "mfma", "achieved": round(g1_tflops, 2),
                      "peak": PEAK_MFMA_FP4_TFLOPS, "unit": "TFLOP/s", "frac": round(g1_tflops / PEAK_MFMA_FP4_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((a.shape, a.tokens)), "avg_launch_ms": round(g1_ms, 4)},
+                     "traffic": MEASURED_TRAFFIC.get((a.shape, a.tokens)), "avg_launch_ms": round(g1_ms, 4),
+                     # the other roof of the same kernel (its algorithmic bytes against the HBM peak)
+                     "hbm_achieved_gbps": round(w["bytes_stage1"] / (g1_ms * 1e-3) / 1e9, 1),
+                     "hbm_frac": round(w["bytes_stage1"] / (g1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)},
         "decode": {"tokens": a.decode_tokens, "ms_per_step": round(dec["ms"], 4), "experts_hit": dw["e_hit"],
                    "hbm_gbps": round(dec_gbps, 1), "frac_of_hbm_peak": round(dec_gbps / PEAK_HBM_GBPS, 4),
                    "tflops": round(dw["flops"] / (dec["ms"] * 1e-3) / 1e12, 2),
