@@ -72,3 +72,15 @@ def test_pad_layer_weights_is_exact():
     # already aligned: returned unchanged
     same = pm.pad_layer_weights(t(w1q), t(w1s), t(w2q), t(w2s), multiple=32)
     assert same[0].data_ptr() == t(w1q).data_ptr() and same[6:] == (0, 0)
+
+
+def test_row_block_heuristic():
+    """smallest of 16 / 32 / 64 / 128 that holds twice the mean rows per expert"""
+    from pyhip_amd.fused_moe import pick_block_m
+    assert pick_block_m(16, 8, 256) == 16            # 0.5 rows per expert
+    assert pick_block_m(256, 8, 256) == 16           # 8
+    assert pick_block_m(512, 8, 256) == 32           # 16
+    assert pick_block_m(1024, 8, 256) == 64          # 32
+    assert pick_block_m(2048, 8, 256) == 128         # 64
+    assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
+    assert pick_block_m(1, 2, 8) == 16 and pick_block_m(4096, 2, 8) == 128
