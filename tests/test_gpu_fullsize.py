@@ -30,7 +30,7 @@ def _run(W, hidden, tw, ti, **kw):
     return fused_moe(hidden, W["w1"], W["w2"], tw, ti, w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], **kw)
 
 
-@pytest.mark.parametrize("T,method", [(16, "w4a16"), (16, "a4w4"), (1024, "a4w4"), (8192, "a4w4")])
+@pytest.mark.parametrize("T,method", [(16, "w4a16"), (16, "a4w4"), (1024, "a4w4"), (8192, "a4w4"), (32768, "a4w4")])
 def test_sampled_experts_and_properties(layer, T, method):
     from pyhip_amd import mxfp4 as pm, workloads
     W = layer
