@@ -740,10 +740,11 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
         g.sched = nullptr;   // a single K-group per tile: no room to prefetch across tiles, one tile per workgroup
     if(g.sched)
     {
-        // persistent: fill every CU at the kernel's occupancy (2 workgroups per CU)
+        // persistent: two workgroups per CU (one for 256-row tiles).  Small tiles would fit three or four; measured,
+        // that changes nothing: they are bound by the weight stream
         int dev = 0, cus = 256;
         if(hipGetDevice(&dev) == hipSuccess)
-            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
