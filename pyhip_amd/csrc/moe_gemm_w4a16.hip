@@ -86,6 +86,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     const uint16_t* ap[MT];
     bool ok[MT];
     u32 ids[MT];
+    const int tok0 = STAGE == 1 ? (int)(g.sorted_ids[m_blk * BM] & 0xFFFFFFu) : 0;
 #pragma unroll
     for(int mt = 0; mt < MT; mt++)
     {
@@ -93,7 +94,10 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
         ids[mt]      = g.sorted_ids[p];
         const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
         ok[mt]       = slot < g.topk && tok < g.T;
-        const size_t row = STAGE == 1 ? (size_t)(ok[mt] ? tok : 0) : (size_t)p;
+        // padding rows compute nothing that is stored: they all read the row of the block's first position, which
+        // always holds a routed row and is read anyway, so the loads coalesce and a sparsely filled block does
+        // not pull 16 distinct rows through the L2 per K-step
+        const size_t row = STAGE == 1 ? (size_t)(ok[mt] ? tok : tok0) : (size_t)(ok[mt] ? p : m_blk * BM);
         ap[mt]       = g.a + row * g.K + kb * 32;
     }
 
