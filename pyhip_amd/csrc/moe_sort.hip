@@ -12,13 +12,15 @@
 //   workgroup) + (#pairs of e earlier in this wave's chunk).
 //
 // Three launches for large inputs (histogram -> scan -> scatter) and one single-workgroup
-// launch for decode-sized inputs.
+// launch for small inputs.
 #include "common.h"
 
 #define SORT_THREADS 256
 #define SORT_WAVES (SORT_THREADS / WAVE)
 #define SMALL_THREADS 1024
 #define SMALL_WAVES (SMALL_THREADS / WAVE)
+#define SMALL_GROUPS 2      // groups of 64 pairs a wave of the single-workgroup sort holds in registers
+#define SORT_GROUPS 4       // the same for a wave of the multi-workgroup sort
 #define EXPERT_FILL 0xFFFFFFFFu
 
 struct SortArgs
@@ -54,57 +56,107 @@ __device__ __forceinline__ int wave_chunk(int pairs, int total_waves)
     return (c + WAVE - 1) / WAVE * WAVE;
 }
 
-// histogram of the pairs [beg, end) into h[E] (LDS), counting only kept experts
-__device__ __forceinline__ void wave_hist(const SortArgs& a, u32* h, int beg, int end)
+// Up to NG groups of 64 consecutive pairs of one wave, held in registers: all their loads are in flight together
+// (a loop of load -> use -> load pays one memory round trip per group), and the scatter reuses what the
+// histogram loaded.  e < 0 marks a pair that is dropped (out of range, masked expert, past the end).
+template <int NG>
+struct WavePairs
 {
-    for(int i = beg + lane_id(); i < end; i += WAVE)
-    {
-        int e = a.topk_ids[i];
-        if(e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0))
-            atomicAdd(&h[e], 1u);
-    }
-}
+    int e[NG];
+    float w[NG];
 
-// writes the pairs [beg, end) to their final positions; base[e] (LDS, private to this wave) is the
-// position of the wave's first pair of expert e and is advanced as groups are consumed.  Within a
-// group of 64 pairs every lane finds the lanes that hold the same expert from one ballot per bit of
-// the expert id (a constant number of steps, however many distinct experts the group holds); its rank
-// among them gives the position, and the lowest such lane advances base[e].
-__device__ __forceinline__ void wave_scatter(const SortArgs& a, u32* base, int beg, int end)
-{
-    const int lane  = lane_id();
-    const u64 lt    = (1ull << lane) - 1ull;
-    const int nbits = 32 - __builtin_clz((unsigned)(a.E > 1 ? a.E - 1 : 1));
-    for(int g = beg; g < end; g += WAVE)
+    // pairs [beg, min(end, beg + NG*64))
+    __device__ __forceinline__ void load(const SortArgs& a, int beg, int end, bool with_weights)
     {
-        int i     = g + lane;
-        int e     = -1;
-        float w   = 0.f;
-        if(i < end)
+        const int lane = lane_id();
+#pragma unroll
+        for(int g = 0; g < NG; g++)
         {
-            e = a.topk_ids[i];
-            w = a.topk_w[i];
+            const int i = beg + g * WAVE + lane;
+            e[g]        = i < end ? a.topk_ids[i] : -1;
+            w[g]        = (with_weights && i < end) ? a.topk_w[i] : 0.f;
         }
-        const bool keep = e >= 0 && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
-        u64 m           = __ballot(keep);
-        for(int b = 0; b < nbits; b++)
+#pragma unroll
+        for(int g = 0; g < NG; g++)
         {
-            const bool bit = (e >> b) & 1;
-            const u64 bal  = __ballot(keep && bit);
-            m &= bit ? bal : ~bal;
+            if(e[g] >= a.E)
+                e[g] = -1;
+            if(a.expert_mask && e[g] >= 0 && a.expert_mask[e[g]] == 0)
+                e[g] = -1;
         }
-        if(keep)
-        {
-            const u32 pos     = base[e] + (u32)__popcll(m & lt);
-            const u32 tok     = (u32)(i / a.k);
-            const u32 slot    = (u32)(i - (int)tok * a.k);
-            a.sorted_ids[pos] = (slot << 24) | tok;
-            a.sorted_w[pos]   = w;
-        }
-        if(keep && (m & lt) == 0)       // lowest lane of its expert; every lane above has read base[e] already
-            base[e] += (u32)__popcll(m);
     }
-}
+
+    // histogram into h[E] (LDS) shared with other waves
+    __device__ __forceinline__ void hist_atomic(u32* h) const
+    {
+#pragma unroll
+        for(int g = 0; g < NG; g++)
+            if(e[g] >= 0)
+                atomicAdd(&h[e[g]], 1u);
+    }
+
+    // Within a group of 64 pairs every lane finds the lanes that hold the same expert from one ballot per bit of
+    // the expert id (a constant number of steps, however many distinct experts the group holds).  Kept per group:
+    // the lane's rank among them (bits 0-7), their number (bits 8-15) and whether the lane is the lowest (bit 16).
+    u32 rc[NG];
+    __device__ __forceinline__ void match(const SortArgs& a, int beg, int end)
+    {
+        const int lane  = lane_id();
+        const u64 lt    = (1ull << lane) - 1ull;
+        const int nbits = 32 - __builtin_clz((unsigned)(a.E > 1 ? a.E - 1 : 1));
+#pragma unroll
+        for(int g = 0; g < NG; g++)
+        {
+            rc[g] = 0;
+            if(beg + g * WAVE >= end)      // uniform
+                continue;
+            const bool keep = e[g] >= 0;
+            u64 m           = __ballot(keep);
+            for(int b = 0; b < nbits; b++)
+            {
+                const bool bit = (e[g] >> b) & 1;
+                const u64 bal  = __ballot(keep && bit);
+                m &= bit ? bal : ~bal;
+            }
+            rc[g] = (u32)__popcll(m & lt) | ((u32)__popcll(m) << 8) | ((m & lt) == 0 ? 1u << 16 : 0u);
+        }
+    }
+
+    // histogram into h[E] (LDS) private to this wave, after match(): the lowest lane of every expert adds the count
+    // (no atomics: the experts of a group are distinct addresses, and a wave's LDS operations execute in order)
+    __device__ __forceinline__ void hist_private(u32* h) const
+    {
+#pragma unroll
+        for(int g = 0; g < NG; g++)
+            if(e[g] >= 0 && (rc[g] >> 16))
+                h[e[g]] += (rc[g] >> 8) & 0xFFu;
+    }
+
+    // after match(): writes the pairs to their final positions; base[e] (LDS, private to this wave) is the position
+    // of the wave's first pair of expert e and is advanced by the lowest lane as groups are consumed
+    __device__ __forceinline__ void scatter(const SortArgs& a, u32* base, int beg, int end) const
+    {
+        const int lane = lane_id();
+#pragma unroll
+        for(int g = 0; g < NG; g++)
+        {
+            if(beg + g * WAVE >= end)      // uniform
+                break;
+            const int i = beg + g * WAVE + lane;
+            if(e[g] >= 0)
+            {
+                const u32 b0      = base[e[g]];
+                const u32 pos     = b0 + (rc[g] & 0xFFu);
+                const u32 tok     = (u32)(i / a.k);
+                const u32 slot    = (u32)(i - (int)tok * a.k);
+                a.sorted_ids[pos] = (slot << 24) | tok;
+                a.sorted_w[pos]   = w[g];
+                if(rc[g] >> 16)                 // every lane of this expert has read base[e] above (one instruction)
+                    base[e[g]] = b0 + ((rc[g] >> 8) & 0xFFu);
+            }
+        }
+    }
+};
 
 // per-expert padded offsets from per-expert totals; one workgroup, any thread count that is a
 // multiple of 64.  tot[e] in, off[e] (exclusive prefix of padded sizes) and lid[e] out; returns
@@ -163,33 +215,32 @@ __device__ __forceinline__ u32 expert_offsets(const SortArgs& a, const u32* tot,
     return run_pad;
 }
 
-// padding entries of every expert's run, the tail past the padded total, the block -> expert
-// table and num_valid.  Touches no position that holds a real pair, so it may run concurrently
-// with the scatter.
-__device__ __forceinline__ void fill_outputs(const SortArgs& a, const u32* tot, const u32* off,
-                                             const u32* lid, u32 padded_total, int T, int tid, int nthreads)
+// Every position of sorted_ids / sorted_weights gets the padding entry.  Depends on nothing the sort computes, so
+// it is issued first and overlaps the loads of the pairs; the scatter overwrites the positions that hold pairs
+// and must be ordered after it (a later launch, or a device-scope fence and a barrier in between).
+__device__ __forceinline__ void fill_padding(const SortArgs& a, int T, u32 tid, u32 nthreads)
 {
     const u32 pad_id = ((u32)a.k << 24) | ((u32)T & 0xFFFFFFu);
     const u32 n      = (u32)a.n_blk * (u32)a.Bm;
-    const int nwaves = nthreads / WAVE, wave = tid / WAVE, lane = tid % WAVE;
-    for(int e = wave; e < a.E; e += nwaves)
-    {
-        if(tot[e] == 0 || (a.expert_mask && a.expert_mask[e] == 0))
-            continue;
-        u32 beg = off[e] + tot[e];
-        u32 end = off[e] + (tot[e] + a.Bm - 1) / a.Bm * a.Bm;
-        for(u32 p = beg + lane; p < end; p += WAVE)
-        {
-            a.sorted_ids[p] = pad_id;
-            a.sorted_w[p]   = 0.f;
-        }
-        for(u32 b = off[e] / a.Bm + lane; b < end / a.Bm; b += WAVE)
-            a.sorted_e[b] = lid[e];
-    }
-    for(u32 p = padded_total + tid; p < n; p += nthreads)
+    for(u32 p = tid; p < n; p += nthreads)
     {
         a.sorted_ids[p] = pad_id;
         a.sorted_w[p]   = 0.f;
+    }
+}
+
+// the block -> expert table and num_valid; one workgroup, 16 lanes share the blocks of an expert
+__device__ __forceinline__ void fill_blocks(const SortArgs& a, const u32* tot, const u32* off, const u32* lid,
+                                            u32 padded_total, int T)
+{
+    const u32 tid = threadIdx.x, nthreads = blockDim.x;
+    for(u32 e = tid / 16; e < (u32)a.E; e += nthreads / 16)
+    {
+        if(tot[e] == 0 || (a.expert_mask && a.expert_mask[e] == 0))
+            continue;
+        const u32 b0 = off[e] / a.Bm, b1 = b0 + (tot[e] + a.Bm - 1) / a.Bm;
+        for(u32 b = b0 + tid % 16; b < b1; b += 16)
+            a.sorted_e[b] = lid[e];
     }
     for(u32 b = padded_total / a.Bm + tid; b < (u32)a.n_blk; b += nthreads)
         a.sorted_e[b] = EXPERT_FILL;
@@ -243,7 +294,7 @@ __device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot
 }
 
 // ---------------------------------------------------------------------------------------------
-// single workgroup: everything in one launch (decode-sized inputs)
+// single workgroup: everything in one launch (up to SMALL_GROUPS * 64 pairs per wave)
 // LDS: whist[SMALL_WAVES][E] | tot[E] | off[E] | lid[E] | scratch[2*SMALL_WAVES]
 extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a)
 {
@@ -259,10 +310,14 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kerne
     const int cv    = wave_chunk(pairs, SMALL_WAVES);
     const int beg   = min(pairs, wave * cv), end = min(pairs, beg + cv);
 
+    WavePairs<SMALL_GROUPS> wp;
+    wp.load(a, beg, end, true);
+    fill_padding(a, T, threadIdx.x, SMALL_THREADS);
     for(int i = threadIdx.x; i < SMALL_WAVES * a.E; i += SMALL_THREADS)
         whist[i] = 0;
     __syncthreads();
-    wave_hist(a, whist + wave * a.E, beg, end);
+    wp.match(a, beg, end);
+    wp.hist_private(whist + wave * a.E);
     __syncthreads();
     // exclusive prefix over waves, per expert
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
@@ -278,17 +333,20 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kerne
     }
     __syncthreads();
     u32 padded_total = expert_offsets(a, tot, off, lid, scratch);
-    fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+    fill_blocks(a, tot, off, lid, padded_total, T);
     write_schedule(a, tot, off, lid);
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         for(int w = 0; w < SMALL_WAVES; w++)
             whist[w * a.E + e] += off[e];
+    // the padding entries have landed (a store leaves the counter when the L2 has it) before any wave of this
+    // workgroup, which shares that L2, writes a pair over them
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    wave_scatter(a, whist + wave * a.E, beg, end);
+    wp.scatter(a, whist + wave * a.E, beg, end);
 }
 
 // ---------------------------------------------------------------------------------------------
-// large inputs, launch 1 of 3: per-workgroup histogram -> ws[g][E]
+// large inputs, launch 1 of 3: per-workgroup histogram -> ws[g][E]; padding entries everywhere
 extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_hist_kernel(SortArgs a)
 {
     extern __shared__ u32 lds[];
@@ -297,16 +355,22 @@ extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_hist_kernel(
     const int cv    = wave_chunk(pairs, a.G * SORT_WAVES);
     const int wid   = blockIdx.x * SORT_WAVES + threadIdx.x / WAVE;
     const int beg   = min(pairs, wid * cv), end = min(pairs, beg + cv);
+    fill_padding(a, T, blockIdx.x * SORT_THREADS + threadIdx.x, gridDim.x * SORT_THREADS);
     for(int i = threadIdx.x; i < a.E; i += SORT_THREADS)
         lds[i] = 0;
     __syncthreads();
-    wave_hist(a, lds, beg, end);
+    WavePairs<SORT_GROUPS> wp;
+    for(int s = beg; s < end; s += SORT_GROUPS * WAVE)
+    {
+        wp.load(a, s, end, false);
+        wp.hist_atomic(lds);
+    }
     __syncthreads();
     for(int i = threadIdx.x; i < a.E; i += SORT_THREADS)
         a.ws[(size_t)blockIdx.x * a.E + i] = lds[i];
 }
 
-// launch 2 of 3 (one workgroup): ws[g][e] -> exclusive prefix over g; offsets; padding; tables
+// launch 2 of 3 (one workgroup): ws[g][e] -> exclusive prefix over g; offsets; tables
 // LDS: tot[E] | off[E] | lid[E] | scratch
 extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel(SortArgs a)
 {
@@ -340,7 +404,7 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel
     u32* g_off       = a.ws + (size_t)a.G * a.E;
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         g_off[e] = off[e];
-    fill_outputs(a, tot, off, lid, padded_total, T, threadIdx.x, SMALL_THREADS);
+    fill_blocks(a, tot, off, lid, padded_total, T);
     write_schedule(a, tot, off, lid);
 }
 
@@ -357,7 +421,14 @@ extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_scatter_kern
     for(int i = threadIdx.x; i < SORT_WAVES * a.E; i += SORT_THREADS)
         lds[i] = 0;
     __syncthreads();
-    wave_hist(a, lds + wave * a.E, beg, end);
+    WavePairs<SORT_GROUPS> wp;
+    const bool once = end - beg <= SORT_GROUPS * WAVE;      // then the registers still hold the chunk for the scatter
+    for(int s = beg; s < end; s += SORT_GROUPS * WAVE)
+    {
+        wp.load(a, s, end, true);
+        wp.match(a, s, end);
+        wp.hist_private(lds + wave * a.E);
+    }
     __syncthreads();
     const u32* g_off = a.ws + (size_t)a.G * a.E;
     for(int e = threadIdx.x; e < a.E; e += SORT_THREADS)
@@ -371,7 +442,15 @@ extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_scatter_kern
         }
     }
     __syncthreads();
-    wave_scatter(a, lds + wave * a.E, beg, end);
+    for(int s = beg; s < end; s += SORT_GROUPS * WAVE)
+    {
+        if(!once)
+        {
+            wp.load(a, s, end, true);
+            wp.match(a, s, end);
+        }
+        wp.scatter(a, lds + wave * a.E, s, end);
+    }
 }
 
 // zero fill of the layer output buffer the reference's sorter hands back
@@ -386,7 +465,7 @@ extern "C" __global__ void moe_zero_kernel(uint4* p, size_t n16, unsigned char* 
 }
 
 // ---------------------------------------------------------------------------------------------
-#define SMALL_PAIRS_MAX 4096
+#define SMALL_PAIRS_MAX (SMALL_WAVES * SMALL_GROUPS * WAVE)
 #define MAX_EXPERTS 2048
 
 static int sort_groups(int64_t pairs)

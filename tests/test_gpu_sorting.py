@@ -37,8 +37,12 @@ def _run(ids, w, E, Bm, mask=None, nloc=None):
 @pytest.mark.parametrize("T,k,E,Bm,skew", [
     (1, 1, 1, 16, False), (1, 8, 256, 16, False), (16, 8, 256, 16, False), (64, 2, 8, 32, False),
     (33, 8, 256, 32, True), (7, 4, 128, 64, False), (200, 8, 32, 64, True), (129, 2, 8, 128, False),
-    (512, 8, 256, 128, True),              # 4096 pairs: the largest single-workgroup case
-    (513, 8, 256, 128, True),              # first multi-launch case
+    (512, 8, 256, 128, True), (513, 8, 256, 128, True),
+    (256, 8, 256, 64, True),               # 2048 pairs: the largest single-workgroup case
+    (257, 8, 256, 64, True),               # first multi-launch case
+    (1024, 8, 256, 64, True), (1025, 8, 256, 64, True),
+    (4097, 2, 8, 16, False), (2048, 4, 1024, 16, True),
+    (40000, 8, 64, 32, True),              # waves of the multi-launch sort take more than one register-load of pairs
     (4096, 2, 8, 256, False), (8192, 8, 256, 256, True), (3000, 4, 128, 16, True), (5000, 20, 400, 32, False),
 ])
 def test_sort_matches_oracle(T, k, E, Bm, skew):
@@ -46,7 +50,7 @@ def test_sort_matches_oracle(T, k, E, Bm, skew):
     _run(_ids(rng, T, k, E, skew), rng.random((T, k), dtype=np.float32), E, Bm)
 
 
-@pytest.mark.parametrize("T,k,E,Bm", [(40, 4, 16, 16), (2000, 8, 64, 32)])
+@pytest.mark.parametrize("T,k,E,Bm", [(40, 4, 16, 16), (700, 8, 64, 32), (2000, 8, 64, 32), (50000, 6, 64, 32)])
 def test_sort_expert_mask_and_local_tokens(T, k, E, Bm):
     rng = np.random.default_rng(T)
     ids, w = _ids(rng, T, k, E, False), rng.random((T, k), dtype=np.float32)
