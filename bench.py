@@ -7,6 +7,8 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
   value     TFLOP/s of the whole layer at --tokens (default 8192), FLOPs = 6*T*k*I*H
   decode    the same layer at --decode-tokens (default 16): ms, HBM GB/s on algorithmic bytes (method="auto":
             bf16 activations x MXFP4 weights at this size)
+            bf16 activations x MXFP4 weights at this size); graph_replay_ms_per_step is the same call captured in
+            a HIP graph and replayed
   decode_a4w4  the same with MXFP4 activations forced (method="a4w4")
   roofline  the dominant kernel (stage-1 gate_up GEMM) of the primary workload, timed with events
             recorded around it inside the timed steps
@@ -75,6 +77,27 @@ def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, metho
                 out=out)
 
 
+def graph_replay_ms(torch, fused_moe, W, res, steps, block_m, method="auto"):
+    """the same call captured once in a HIP graph and replayed: what a serving loop that captures its decode step
+    pays per layer (no host work between the launches)"""
+    kw = dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
+              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"],
+              method=method)
+    args = (res["hidden"], W["w1"], W["w2"], res["topk_w"], res["topk_ids"])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fused_moe(*args, **kw)
+    for _ in range(5):
+        graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, res["out"]), "graph replay differs from the eager result"
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 class LazyExperts:
     """expert-indexed view that copies one expert's (de-shuffled) bytes from the device on demand"""
 
@@ -137,6 +160,7 @@ def main():
     main_res = run_config(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m)
     dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
     dec4 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
+    dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
 
     if a.calibrate_copy:
         src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
@@ -174,6 +198,7 @@ def main():
                    "hbm_gbps": round(dec_gbps, 1), "frac_of_hbm_peak": round(dec_gbps / PEAK_HBM_GBPS, 4),
                    "tflops": round(dw["flops"] / (dec["ms"] * 1e-3) / 1e12, 2),
                    "stage_ms": {k: round(v, 4) for k, v in dec["stage_ms"].items()},
+                   "graph_replay_ms_per_step": round(dec_graph_ms, 4),
                    "roofline": {"kernel": "moe_gemm_w4a16_kernel<1,1> (gate_up, bf16 activations)", "bound": "hbm",
                                 "achieved": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                                 "unit": "GB/s",
