@@ -97,10 +97,13 @@ __device__ __forceinline__ v4i make_rsrc(const void* p, u32 bytes)
     return (v4i){(int)(u32)a, (int)((a >> 32) & 0xFFFFu), (int)bytes, 0x00020000};
 }
 // address = rsrc.base + voff + soff + IMM (IMM < 4096); only voff + IMM is range-checked
-template <int IMM = 0>
+template <int IMM = 0, bool NT = false>
 __device__ __forceinline__ void vm_load_b128(v4i& dst, int voff, v4i rsrc, int soff)
 {
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+    if(NT)      // streamed once: the line is the first to go when the L2 needs room
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4 nt" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+    else
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
 }
 template <int IMM = 0>
 __device__ __forceinline__ void vm_load_b32(int& dst, int voff, v4i rsrc, int soff)
@@ -183,7 +186,9 @@ struct TileId
 // the memory pipeline never drains between tiles.  One barrier per K-group (512 K elements).  Everything
 // a tile boundary needs (schedule tables, sorted ids, routing weights) is read from LDS, so no wait on the
 // vector-memory counter ever covers the prefetches in flight.
-template <int STAGE, int MT, int ACT>
+// NT: the weight loads are marked non-temporal (the launch decides: set when nearly every expert has a single row
+// block, so that no other workgroup reads the same weight tile)
+template <int STAGE, int MT, int ACT, bool NT>
 __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
@@ -411,7 +416,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     };
     auto load_wtile = [&](auto U, auto J, int kt) __attribute__((always_inline)) {
         constexpr int u = decltype(U)::value, j = decltype(J)::value;
-        vm_load_b128<0>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
+        vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
     };
     auto load_wtiles = [&](auto U, int kt) __attribute__((always_inline)) {
         static_for<4>([&](auto J) __attribute__((always_inline)) { load_wtile(U, J, kt); });
@@ -749,13 +754,27 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
     dim3 grid(nwg), block(GEMM_THREADS);
+    // Non-temporal weight loads when the routed rows per expert (T * topk / E on average) stay under three quarters
+    // of a row block: nearly every expert then has one block, each weight tile one reader, and lines that are
+    // dropped first leave the L2 to the activations.  With several blocks per expert the readers of a tile find
+    // each other's lines in the L2 and the marking would throw that away.
+    const bool nt = (int64_t)g.T * g.topk * 4 <= (int64_t)g.E * block_m * 3;
     // ACT (0 SiLU * up, 1 clamped SwiGLU) only exists for the gate_up stage
+#define GEMM_LAUNCH(MTV, ACTV, NTV) \
+    hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, ACTV, NTV>), grid, block, 0, stream, g)
 #define GEMM_CASE(BM, MTV)                                                                                         \
     case BM:                                                                                                       \
         if(STAGE == 1 && act == 1)                                                                                 \
-            hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, STAGE == 1 ? 1 : 0>), grid, block, 0, stream, g); \
+        {                                                                                                          \
+            if(MTV <= 8 && nt)                                                                                     \
+                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), (MTV <= 8));                                                \
+            else                                                                                                   \
+                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), false);                                                     \
+        }                                                                                                          \
+        else if(MTV <= 8 && nt)                                                                                    \
+            GEMM_LAUNCH(MTV, 0, (MTV <= 8));                                                                       \
         else                                                                                                       \
-            hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, 0>), grid, block, 0, stream, g);                  \
+            GEMM_LAUNCH(MTV, 0, false);                                                                            \
         break;
     switch(block_m)
     {
@@ -763,6 +782,7 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
     default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256}", block_m); return PYHIP_ERR_INVALID;
     }
 #undef GEMM_CASE
+#undef GEMM_LAUNCH
     PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel");
     return PYHIP_OK;
 }

@@ -42,6 +42,20 @@ def pick_block_m(tokens, topk, experts):
     return 128
 
 
+def pick_w4a16(tokens, topk, experts, hidden):
+    """``method="auto"``: True selects the bf16-activation kernels (the reference switches to its w4a16 split-K
+    kernel for few tokens, src/contrib/moe.py:362-787).  They win in two regimes (measured on all five benchmark
+    shapes): fewer than 0.75 routed rows per expert on average (DS-V3 T = 16: 0.40 against 0.42 ms; from one row per
+    expert on the MXFP4-activation kernels stream faster), and layers with so few experts that the down GEMM of the
+    MXFP4-activation path, one workgroup per (row block, 256 output channels), cannot fill the GPU while the
+    bf16-activation kernel splits K over four times as many workgroups (Mixtral shape up to 8 rows per expert,
+    T = 1: 0.068 against 0.109 ms)."""
+    pairs = tokens * topk
+    sparse = 4 * pairs <= 3 * experts
+    few_tiles = min(pairs, experts) * (hidden // 256) < 512 and pairs <= 8 * experts
+    return sparse or few_tiles
+
+
 def act_quant_mxfp4(x, rows_limit=None):
     """bf16 [rows, K] -> (uint8 [rows, K/2], uint8 [rows, ceil(K/512)*16]) in the GEMM's A-operand layout."""
     lib = _lib.load()
@@ -134,9 +148,8 @@ def fused_moe(
     topk_ids = topk_ids.to(torch.int32).contiguous()
     topk_weight = topk_weight.to(torch.float32).contiguous()
     assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
-    # "auto" (and the reference's "jit" / "gluon", which name its own back ends): bf16 activations while the
-    # layer only streams weights (at most 2 routed rows per expert on average), MXFP4 activations above that
-    w4a16 = method == "w4a16" or (method != "a4w4" and T * k <= 2 * global_E)
+    # "auto" (and the reference's "jit" / "gluon", which name its own back ends): see pick_w4a16
+    w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, k, global_E, H))
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
     if w4a16:
         bm = min(bm, 64)

@@ -22,8 +22,8 @@ def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(tmp_path):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout[-2000:]
     text = out.read_text()
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dEEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", text, re.S | re.M)
-    assert len(kernels) == 15, "expected (gate_up x two activations + down) x five tile heights"
+    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", text, re.S | re.M)
+    assert len(kernels) == 27, "expected (gate_up x two activations + down) x (four tile heights x two load policies + the 256-row tile)"
     for name, body in kernels:
         inside = False
         hand = {"mfma": 0, "read": 0, "write": 0}
@@ -60,8 +60,8 @@ def test_no_vector_written_scalar_register_is_read_too_early_by_vector_memory(tm
     cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout[-2000:]
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dEEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
-    assert len(kernels) == 15
+    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
+    assert len(kernels) == 27
     for name, body in kernels:
         ins = list(_instructions(body))
         for i, line in enumerate(ins):
@@ -102,8 +102,8 @@ def test_compiler_never_copies_a_register_with_a_load_in_flight(tmp_path):
     cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout[-2000:]
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dEEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
-    assert len(kernels) == 15
+    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
+    assert len(kernels) == 27
     for name, body in kernels:
         # Walk the kernel text: a register is "loaded" from the inline-assembly load that writes it until the
         # compiler's own code overwrites it with something else.  Values loaded that way are consumed by

@@ -84,3 +84,15 @@ def test_row_block_heuristic():
     assert pick_block_m(2048, 8, 256) == 128         # 64
     assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
     assert pick_block_m(1, 2, 8) == 16 and pick_block_m(4096, 2, 8) == 128
+
+
+def test_auto_method_rule():
+    """bf16 activations below 0.75 routed rows per expert, or while few experts leave the down GEMM short of tiles"""
+    from pyhip_amd.fused_moe import pick_w4a16
+    assert pick_w4a16(16, 8, 256, 7168) and pick_w4a16(24, 8, 256, 7168)          # DS-V3: 0.5 and 0.75 rows per expert
+    assert not pick_w4a16(32, 8, 256, 7168) and not pick_w4a16(8192, 8, 256, 7168)
+    assert pick_w4a16(8, 8, 128, 4096) and not pick_w4a16(16, 8, 128, 4096)       # Qwen3
+    assert pick_w4a16(16, 4, 128, 3072) and not pick_w4a16(32, 4, 128, 3072)      # gpt-oss, padded width
+    assert pick_w4a16(1, 2, 8, 4096) and pick_w4a16(32, 2, 8, 4096)               # Mixtral: 8 experts x 16 tiles
+    assert not pick_w4a16(48, 2, 8, 4096) and not pick_w4a16(4096, 2, 8, 4096)
+    assert not pick_w4a16(64, 2, 8, 1024)                                         # the tiny shape at 16 rows per expert
