@@ -762,19 +762,19 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
     // ACT (0 SiLU * up, 1 clamped SwiGLU) only exists for the gate_up stage
 #define GEMM_LAUNCH(MTV, ACTV, NTV) \
     hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, ACTV, NTV>), grid, block, 0, stream, g)
-#define GEMM_CASE(BM, MTV)                                                                                         \
-    case BM:                                                                                                       \
-        if(STAGE == 1 && act == 1)                                                                                 \
-        {                                                                                                          \
-            if(MTV <= 8 && nt)                                                                                     \
-                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), (MTV <= 8));                                                \
-            else                                                                                                   \
-                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), false);                                                     \
-        }                                                                                                          \
-        else if(MTV <= 8 && nt)                                                                                    \
-            GEMM_LAUNCH(MTV, 0, (MTV <= 8));                                                                       \
-        else                                                                                                       \
-            GEMM_LAUNCH(MTV, 0, false);                                                                            \
+#define GEMM_CASE(BM, MTV)                                       \
+    case BM:                                                     \
+        if(STAGE == 1 && act == 1)                               \
+        {                                                        \
+            if(nt)                                               \
+                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), true);    \
+            else                                                 \
+                GEMM_LAUNCH(MTV, (STAGE == 1 ? 1 : 0), false);   \
+        }                                                        \
+        else if(nt)                                              \
+            GEMM_LAUNCH(MTV, 0, true);                           \
+        else                                                     \
+            GEMM_LAUNCH(MTV, 0, false);                          \
         break;
     switch(block_m)
     {

@@ -29,16 +29,24 @@ def _as_u8(t):
     return t if t.dtype == torch.uint8 else t.view(torch.uint8)
 
 
-def pick_block_m(tokens, topk, experts):
+def pick_block_m(tokens, topk, experts, hidden=0):
     """M-tile (= sort block size): the smallest tile that holds TWICE the expected rows per expert.  Every extra
     row block of an expert streams the expert's weights once more, and routing is uneven enough that a tile of just
     the mean size overflows for about half of the experts; the rows a larger tile leaves empty fetch nothing
     (measured on the DS-V3 shape: T = 1024: 64-row tiles 1.20 ms against 1.27 ms with 32; T = 2048: 128-row tiles
-    1.27 ms against 1.39 ms with 64)."""
+    1.27 ms against 1.39 ms with 64).
+
+    The 256-row tile (one wave per SIMD, slower per FLOP) is taken where it saves a whole pass over the weights:
+    between 120 and 192 expected rows per expert a 128-row tile needs two blocks for most experts and the 256-row
+    tile one, read with non-temporal loads.  Its long epilogue only pays with a long K loop: DS-V3 (hidden 7168)
+    T = 4096 / 5120 / 6144: 1.55 / 1.65 / 1.72 ms against 1.69 / 2.09 / 1.92 ms; the gpt-oss, Qwen3 and Mixtral shapes
+    (hidden 3072 / 4096) lose 4-13 % with it at the same rows per expert."""
     est = tokens * topk / max(experts, 1)
     for bm in (16, 32, 64):
         if 2 * est <= bm:
             return bm
+    if hidden >= 6144 and 120 <= est <= 192:
+        return 256
     return 128
 
 
@@ -150,7 +158,7 @@ def fused_moe(
     assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
     # "auto" (and the reference's "jit" / "gluon", which name its own back ends): see pick_w4a16
     w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, k, global_E, H))
-    bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E)
+    bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E, H)
     if w4a16:
         bm = min(bm, 64)
     ev = _mark("start")

@@ -12,18 +12,27 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SRC = os.path.join(ROOT, "pyhip_amd", "csrc", "moe_gemm_mxfp4.hip")
+KERNEL_RE = r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel"
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
-def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(tmp_path):
+@pytest.fixture(scope="module")
+def gemm_asm(tmp_path_factory):
+    """the device assembly of the GEMM source, compiled once with the library's own flags"""
+    if shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"):
+        pytest.skip("needs hipcc")
     from pyhip_amd import build
-    out = tmp_path / "gemm.s"
+    out = tmp_path_factory.mktemp("asm") / "gemm.s"
     cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout[-2000:]
     text = out.read_text()
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", text, re.S | re.M)
-    assert len(kernels) == 27, "expected (gate_up x two activations + down) x (four tile heights x two load policies + the 256-row tile)"
+    kernels = re.findall(KERNEL_RE, text, re.S | re.M)
+    assert len(kernels) == 30, "expected (gate_up x two activations + down) x five tile heights x two load policies"
+    return text, kernels
+
+
+def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(gemm_asm):
+    text, kernels = gemm_asm
     for name, body in kernels:
         inside = False
         hand = {"mfma": 0, "read": 0, "write": 0}
@@ -50,18 +59,11 @@ def _instructions(body):
             yield code
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
-def test_no_vector_written_scalar_register_is_read_too_early_by_vector_memory(tmp_path):
+def test_no_vector_written_scalar_register_is_read_too_early_by_vector_memory(gemm_asm):
     """gfx9 hazard: a vector-memory instruction may read a scalar register only 5 wait states after a vector
     instruction (v_readlane / v_readfirstlane) wrote it.  The compiler pads its own instructions but not the
     hand-written ones inside inline assembly, so the generated code of every GEMM kernel is scanned."""
-    from pyhip_amd import build
-    out = tmp_path / "gemm.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert r.returncode == 0, r.stdout[-2000:]
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
-    assert len(kernels) == 27
+    _, kernels = gemm_asm
     for name, body in kernels:
         ins = list(_instructions(body))
         for i, line in enumerate(ins):
@@ -90,20 +92,13 @@ def _vgprs(operand_text):
     return regs
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="needs hipcc")
-def test_compiler_never_copies_a_register_with_a_load_in_flight(tmp_path):
+def test_compiler_never_copies_a_register_with_a_load_in_flight(gemm_asm):
     """The weight tiles and weight scales are loaded by inline assembly long before they are used, and only the
     hand-written waits know when they have arrived.  That holds as long as the compiler leaves those registers
     alone: a copy it inserts (live-range splitting, a join between two instances of a loop body) would read a
     register whose load is still in flight.  Check: outside the inline-assembly regions no instruction of a GEMM
     kernel reads or writes a register that an inline-assembly load writes to."""
-    from pyhip_amd import build
-    out = tmp_path / "gemm.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert r.returncode == 0, r.stdout[-2000:]
-    kernels = re.findall(r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel", out.read_text(), re.S | re.M)
-    assert len(kernels) == 27
+    _, kernels = gemm_asm
     for name, body in kernels:
         # Walk the kernel text: a register is "loaded" from the inline-assembly load that writes it until the
         # compiler's own code overwrites it with something else.  Values loaded that way are consumed by

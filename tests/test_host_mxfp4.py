@@ -84,6 +84,10 @@ def test_row_block_heuristic():
     assert pick_block_m(2048, 8, 256) == 128         # 64
     assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
     assert pick_block_m(1, 2, 8) == 16 and pick_block_m(4096, 2, 8) == 128
+    # the 256-row tile: 120..192 rows per expert and a long K loop
+    assert pick_block_m(4096, 8, 256, 7168) == 256 and pick_block_m(6144, 8, 256, 7168) == 256
+    assert pick_block_m(3584, 8, 256, 7168) == 128 and pick_block_m(7168, 8, 256, 7168) == 128
+    assert pick_block_m(4096, 4, 128, 3072) == 128 and pick_block_m(2048, 8, 128, 4096) == 128
 
 
 def test_auto_method_rule():
