@@ -106,3 +106,20 @@ def test_tile_heights_agree_bit_for_bit(layer):
     assert torch.isfinite(outs[128].float()).all()
     assert torch.equal(outs[64], outs[128])
     assert torch.equal(outs[256], outs[128])
+
+
+@pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 256))])
+def test_load_policies_agree_bit_for_bit(layer, T, bms):
+    """The launch marks the weight loads non-temporal while the rows per expert stay under three quarters of a row
+    block (T=1024: 32 rows per expert, so the 64-, 128- and 256-row tiles take that instance and the 16- and 32-row
+    tiles the other; T=4096: 128 rows per expert, only the 256-row tile does).  A cache policy must not change a
+    bit of the result."""
+    W = layer
+    from pyhip_amd import workloads
+    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
+    print(f"full-size case {SHAPE} T={T} block_size_M {bms}", flush=True)
+    outs = {bm: _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm) for bm in bms}
+    torch.cuda.synchronize()
+    assert torch.isfinite(outs[bms[0]].float()).all()
+    for bm in bms[1:]:
+        assert torch.equal(outs[bm], outs[bms[0]]), bm
