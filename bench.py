@@ -10,8 +10,9 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
             bf16 activations x MXFP4 weights at this size); graph_replay_ms_per_step is the same call captured in
             a HIP graph and replayed
   decode_a4w4  the same with MXFP4 activations forced (method="a4w4")
+  sweep     the same layer at --sweep-tokens (default 128, 1024, 4096): ms, TFLOP/s and GB/s on algorithmic work
   roofline  the dominant kernel (stage-1 gate_up GEMM) of the primary workload, timed with events
-            recorded around it inside the timed steps
+            recorded around it inside the timed steps (every fourth one)
   cpu_baseline  the CPU oracle (oracle/moe.py) on a bounded sample of the same workload
 """
 import argparse
@@ -43,6 +44,8 @@ def parse():
     ap.add_argument("--shape", default="dsv3")
     ap.add_argument("--tokens", type=int, default=8192)
     ap.add_argument("--decode-tokens", type=int, default=16)
+    ap.add_argument("--sweep-tokens", type=lambda v: [int(x) for x in v.split(",") if x], default=[128, 1024, 4096],
+                    help="further token counts reported in 'sweep' (comma separated; empty = none)")
     ap.add_argument("--block-m", type=int, default=0)
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="target size of the CPU sample; 0 = skip")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
@@ -63,8 +66,9 @@ def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, metho
     torch.cuda.synchronize()
     events = []
     t0 = time.perf_counter()
-    for _ in range(steps):
-        out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, stage_events=events, **kw)
+    for i in range(steps):
+        # stage events on every fourth timed step: recording one costs several microseconds of GPU time
+        out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, stage_events=events if i % 4 == 0 else None, **kw)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     assert torch.isfinite(out.float()).all()
@@ -161,6 +165,16 @@ def main():
     dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
     dec4 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
     dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
+    # the same layer at sizes between the two headline points (method and row block chosen by the operator)
+    sweep = []
+    for t in a.sweep_tokens:
+        r = run_config(torch, fused_moe, W, a.shape, t, a.steps, a.warmup, a.block_m)
+        sweep.append({"tokens": t, "ms_per_step": round(r["ms"], 4),
+                      "tflops": round(r["work"]["flops"] / (r["ms"] * 1e-3) / 1e12, 1),
+                      "frac_of_mfma_peak": round(r["work"]["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_MFMA_FP4_TFLOPS, 4),
+                      "hbm_gbps": round(r["work"]["bytes"] / (r["ms"] * 1e-3) / 1e9, 1),
+                      "frac_of_hbm_peak": round(r["work"]["bytes"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)})
+        del r
 
     if a.calibrate_copy:
         src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
@@ -210,6 +224,7 @@ def main():
                           "hbm_gbps": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9, 1),
                           "frac_of_hbm_peak": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                           "stage_ms": {k: round(v, 4) for k, v in dec4["stage_ms"].items()}}
+    out["sweep"] = sweep
     if a.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds)
     print(json.dumps(out))
