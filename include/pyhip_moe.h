@@ -72,6 +72,18 @@ int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int to
                       uint32_t* num_valid_ids, uint32_t* schedule, void* moe_out, int64_t moe_out_bytes,
                       void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
 
+/* The same sort with the dynamic MXFP4 quantisation of the layer input (pyhip_moe_act_quant_mxfp4 below: x, row
+ * stride, rows, K -> q, scales) carried in the sort's own launches: the two are independent, and the sort has
+ * a single-workgroup phase during which the quantisation runs on the rest of the GPU.  One dispatch less than
+ * calling both; the results are those of the separate calls.  In the reference the two are separate steps as well
+ * (src/contrib/fused_moe.py:283 and tests/contrib/moe/test_moe.py:664-679). */
+int pyhip_moe_sorting_quant(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk, int experts,
+                            int block_size, const int32_t* expert_mask, const int32_t* num_local_tokens,
+                            uint32_t* sorted_ids, float* sorted_weights, uint32_t* sorted_expert_ids,
+                            uint32_t* num_valid_ids, uint32_t* schedule, void* workspace, int64_t workspace_bytes,
+                            const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K, uint8_t* q,
+                            uint8_t* scales, pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Dynamic MXFP4 quantisation of bf16 activations (1x32 blocks, e8m0 scale
  * 2^(floor(log2 amax) - 2), e2m1 round-to-nearest-even).  Replaces

@@ -10,74 +10,46 @@
 //                   byte (kb*4 + i) holds the scale of block (4*i + kb).  The MFMA lane that owns
 //                   K-block kb of a row then reads ONE dword (offset kb*4) and selects the byte of
 //                   K-step i with the instruction's op_sel.
-#include "common.h"
+#include "quant_device.h"
 
 #define QUANT_THREADS 256
 
-// one thread per 32-element block; 16 consecutive threads own one 16-byte scale group
-extern "C" __global__ void __launch_bounds__(QUANT_THREADS)
-    moe_act_quant_mxfp4_kernel(const uint16_t* __restrict__ x, long long ldx, uint8_t* __restrict__ q,
-                               uint8_t* __restrict__ s, long long rows, int K, int SK,
-                               const u32* __restrict__ rows_limit)
+extern "C" __global__ void __launch_bounds__(QUANT_THREADS) moe_act_quant_mxfp4_kernel(QuantArgs a)
 {
-    if(rows_limit)
-    {
-        long long lim = (long long)*rows_limit;
-        rows          = rows < lim ? rows : lim;
-    }
-    const long long id = (long long)blockIdx.x * QUANT_THREADS + threadIdx.x;
-    const long long row = id / SK;
-    const int j         = (int)(id - row * SK);          // block index inside the row (may be padding)
-    if(row >= rows)                                      // whole 16-thread groups leave together
-        return;
-    u32 e8 = 0;
-    if(j * 32 < K)
-    {
-        const uint4* src = (const uint4*)(x + row * ldx + (long long)j * 32);
-        uint4 v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
-        u32 am = 0;
-        am = amax15(am, v0.x); am = amax15(am, v0.y); am = amax15(am, v0.z); am = amax15(am, v0.w);
-        am = amax15(am, v1.x); am = amax15(am, v1.y); am = amax15(am, v1.z); am = amax15(am, v1.w);
-        am = amax15(am, v2.x); am = amax15(am, v2.y); am = amax15(am, v2.z); am = amax15(am, v2.w);
-        am = amax15(am, v3.x); am = amax15(am, v3.y); am = amax15(am, v3.z); am = amax15(am, v3.w);
-        e8        = mx_scale_byte(am);
-        float mul = mx_inv_scale(e8);
-        uint4 o;
-        o.x = cvt8(v0, mul);
-        o.y = cvt8(v1, mul);
-        o.z = cvt8(v2, mul);
-        o.w = cvt8(v3, mul);
-        *(uint4*)(q + row * (long long)(K / 2) + (long long)j * 16) = o;
-    }
-    // 4x4 byte transpose of the 16 scales of this group through lane shuffles
-    const int jj = j & 15;
-    u32 b0 = __shfl(e8, 0 + (jj & 3), 16), b1 = __shfl(e8, 4 + (jj & 3), 16);
-    u32 b2 = __shfl(e8, 8 + (jj & 3), 16), b3 = __shfl(e8, 12 + (jj & 3), 16);
-    if(jj < 4)
-        *(u32*)(s + row * (long long)SK + (j & ~15) + jj * 4) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+    act_quant_block(a, (long long)blockIdx.x * QUANT_THREADS + threadIdx.x);
 }
 
 extern "C" int64_t pyhip_moe_act_scale_stride(int K) { return ((int64_t)K + 511) / 512 * 16; }
+
+int pyhip_make_quant_args(const char* name, const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K,
+                          uint8_t* q, uint8_t* scales, const uint32_t* rows_limit, QuantArgs* out)
+{
+    PYHIP_REQUIRE(x_bf16 && q && scales, "%s: null pointer", name);
+    PYHIP_REQUIRE(K > 0 && K % 32 == 0, "%s: K=%d must be a positive multiple of 32", name, K);
+    PYHIP_REQUIRE(row_stride_elems >= K && row_stride_elems % 8 == 0,
+                  "%s: row stride %lld must be >= K and a multiple of 8 elements", name, (long long)row_stride_elems);
+    PYHIP_REQUIRE(((uintptr_t)x_bf16 % 16) == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)scales % 4) == 0,
+                  "%s: pointers must be 16-byte aligned", name);
+    out->x = (const uint16_t*)x_bf16; out->ldx = (long long)row_stride_elems; out->q = q; out->s = scales;
+    out->rows = rows > 0 ? (long long)rows : 0; out->K = K; out->SK = (int)pyhip_moe_act_scale_stride(K);
+    out->rows_limit = rows_limit;
+    PYHIP_REQUIRE(out->rows * out->SK < (1ll << 40), "%s: too many rows", name);
+    return PYHIP_OK;
+}
 
 extern "C" int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K,
                                          uint8_t* q, uint8_t* scales, const uint32_t* rows_limit,
                                          hipStream_t stream)
 {
-    PYHIP_REQUIRE(x_bf16 && q && scales, "act_quant: null pointer");
-    PYHIP_REQUIRE(K > 0 && K % 32 == 0, "act_quant: K=%d must be a positive multiple of 32", K);
-    PYHIP_REQUIRE(row_stride_elems >= K && row_stride_elems % 8 == 0,
-                  "act_quant: row stride %lld must be >= K and a multiple of 8 elements", (long long)row_stride_elems);
-    PYHIP_REQUIRE(((uintptr_t)x_bf16 % 16) == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)scales % 4) == 0,
-                  "act_quant: pointers must be 16-byte aligned");
-    if(rows <= 0)
+    QuantArgs a;
+    int rc = pyhip_make_quant_args("act_quant", x_bf16, row_stride_elems, rows, K, q, scales, rows_limit, &a);
+    if(rc)
+        return rc;
+    if(a.rows == 0)
         return PYHIP_OK;
-    int SK          = (int)pyhip_moe_act_scale_stride(K);
-    long long total = rows * SK;
-    long long grid  = (total + QUANT_THREADS - 1) / QUANT_THREADS;
+    long long grid = (a.rows * a.SK + QUANT_THREADS - 1) / QUANT_THREADS;
     PYHIP_REQUIRE(grid < (1ll << 31), "act_quant: too many rows");
-    hipLaunchKernelGGL(moe_act_quant_mxfp4_kernel, dim3((unsigned)grid), dim3(QUANT_THREADS), 0, stream,
-                       (const uint16_t*)x_bf16, (long long)row_stride_elems, q, scales, (long long)rows, K, SK,
-                       rows_limit);
+    hipLaunchKernelGGL(moe_act_quant_mxfp4_kernel, dim3((unsigned)grid), dim3(QUANT_THREADS), 0, stream, a);
     PYHIP_CHECK_LAUNCH("moe_act_quant_mxfp4_kernel");
     return PYHIP_OK;
 }

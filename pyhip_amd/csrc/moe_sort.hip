@@ -14,6 +14,7 @@
 // Three launches for large inputs (histogram -> scan -> scatter) and one single-workgroup
 // launch for small inputs.
 #include "common.h"
+#include "quant_device.h"
 
 #define SORT_THREADS 256
 #define SORT_WAVES (SORT_THREADS / WAVE)
@@ -296,8 +297,15 @@ __device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot
 // ---------------------------------------------------------------------------------------------
 // single workgroup: everything in one launch (up to SMALL_GROUPS * 64 pairs per wave)
 // LDS: whist[SMALL_WAVES][E] | tot[E] | off[E] | lid[E] | scratch[2*SMALL_WAVES]
-extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a)
+// Workgroups past the first quantise activations (qa.rows > 0): the input quantisation of the MXFP4-activation
+// path depends on nothing the sort computes, and carrying it in this launch saves a dispatch.
+extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a, QuantArgs qa)
 {
+    if(blockIdx.x > 0)
+    {
+        act_quant_block(qa, (long long)(blockIdx.x - 1) * SMALL_THREADS + threadIdx.x);
+        return;
+    }
     extern __shared__ u32 lds[];
     u32* whist   = lds;
     u32* tot     = whist + SMALL_WAVES * a.E;
@@ -372,8 +380,15 @@ extern "C" __global__ void __launch_bounds__(SORT_THREADS) moe_sort_hist_kernel(
 
 // launch 2 of 3 (one workgroup): ws[g][e] -> exclusive prefix over g; offsets; tables
 // LDS: tot[E] | off[E] | lid[E] | scratch
-extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel(SortArgs a)
+// Workgroups past the first quantise activations, as in the single-workgroup sort: the scan is one workgroup
+// of serial work during which the rest of the GPU would idle.
+extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel(SortArgs a, QuantArgs qa)
 {
+    if(blockIdx.x > 0)
+    {
+        act_quant_block(qa, (long long)(blockIdx.x - 1) * SMALL_THREADS + threadIdx.x);
+        return;
+    }
     extern __shared__ u32 lds[];
     u32* tot     = lds;
     u32* off     = tot + a.E;
@@ -490,12 +505,12 @@ extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, i
 
 extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 8ll * (experts / 8 + 2) + 2ll * experts; }
 
-extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
-                                 int experts, int block_size, const int32_t* expert_mask,
-                                 const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
-                                 uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
-                                 void* moe_out, int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
-                                 hipStream_t stream)
+static int sorting_impl(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
+                        int experts, int block_size, const int32_t* expert_mask,
+                        const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
+                        uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
+                        void* moe_out, int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
+                        QuantArgs qa, hipStream_t stream)
 {
     PYHIP_REQUIRE(topk_ids && topk_weights && sorted_ids && sorted_weights && sorted_expert_ids && num_valid_ids,
                   "moe_sorting: null pointer");
@@ -536,6 +551,10 @@ extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weig
                            (unsigned char*)moe_out + n16 * 16, ntail);
         PYHIP_CHECK_LAUNCH("moe_zero_kernel");
     }
+    // workgroups that quantise, riding on the single-workgroup launch of either path
+    const long long qwork = qa.rows * qa.SK;
+    PYHIP_REQUIRE((qwork + SMALL_THREADS - 1) / SMALL_THREADS < (1ll << 31) - 1, "moe_sorting: too many rows to quantise");
+    const unsigned qblocks = (unsigned)((qwork + SMALL_THREADS - 1) / SMALL_THREADS);
     if(pairs <= SMALL_PAIRS_MAX)
     {
         size_t lds = ((size_t)(SMALL_WAVES + 3) * experts + 2 * SMALL_WAVES + 2) * 4;
@@ -545,18 +564,48 @@ extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weig
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             PYHIP_REQUIRE(e == hipSuccess, "moe_sorting: cannot reserve %zu B of LDS", lds);
         }
-        hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(SMALL_THREADS), lds, stream, a);
+        hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1 + qblocks), dim3(SMALL_THREADS), lds, stream, a, qa);
         PYHIP_CHECK_LAUNCH("moe_sort_small_kernel");
         return PYHIP_OK;
     }
     a.G = sort_groups(pairs);
     hipLaunchKernelGGL(moe_sort_hist_kernel, dim3(a.G), dim3(SORT_THREADS), (size_t)experts * 4, stream, a);
     PYHIP_CHECK_LAUNCH("moe_sort_hist_kernel");
-    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(SMALL_THREADS),
-                       ((size_t)3 * experts + 2 * SMALL_WAVES + 2) * 4, stream, a);
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1 + qblocks), dim3(SMALL_THREADS),
+                       ((size_t)3 * experts + 2 * SMALL_WAVES + 2) * 4, stream, a, qa);
     PYHIP_CHECK_LAUNCH("moe_sort_scan_kernel");
     hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(a.G), dim3(SORT_THREADS), (size_t)SORT_WAVES * experts * 4,
                        stream, a);
     PYHIP_CHECK_LAUNCH("moe_sort_scatter_kernel");
     return PYHIP_OK;
+}
+
+extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
+                                 int experts, int block_size, const int32_t* expert_mask,
+                                 const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
+                                 uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
+                                 void* moe_out, int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
+                                 hipStream_t stream)
+{
+    QuantArgs qa = {};
+    return sorting_impl(topk_ids, topk_weights, tokens, topk, experts, block_size, expert_mask, num_local_tokens,
+                        sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, schedule, moe_out, moe_out_bytes,
+                        workspace, workspace_bytes, qa, stream);
+}
+
+extern "C" int pyhip_moe_sorting_quant(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
+                                       int experts, int block_size, const int32_t* expert_mask,
+                                       const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
+                                       uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
+                                       void* workspace, int64_t workspace_bytes, const void* x_bf16,
+                                       int64_t row_stride_elems, int64_t rows, int K, uint8_t* q, uint8_t* scales,
+                                       hipStream_t stream)
+{
+    QuantArgs qa;
+    int rc = pyhip_make_quant_args("moe_sorting_quant", x_bf16, row_stride_elems, rows, K, q, scales, nullptr, &qa);
+    if(rc)
+        return rc;
+    return sorting_impl(topk_ids, topk_weights, tokens, topk, experts, block_size, expert_mask, num_local_tokens,
+                        sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, schedule, nullptr, 0, workspace,
+                        workspace_bytes, qa, stream);
 }

@@ -162,9 +162,13 @@ def fused_moe(
     if w4a16:
         bm = min(bm, 64)
     ev = _mark("start")
-    sorted_ids, sorted_w, sorted_e, num_valid, _, sched = moe_sorting(
-        topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
-        moe_sorting_dispatch_policy, alloc_moe_out=False, return_schedule=True)
+    # MXFP4-activation path: the input quantisation rides in the sort's launches (independent work, one dispatch less)
+    qin = None
+    if not w4a16:
+        qin = hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous()
+    res = moe_sorting(topk_ids, topk_weight, global_E, H, out_dtype, bm, expert_mask, num_local_tokens,
+                      moe_sorting_dispatch_policy, alloc_moe_out=False, return_schedule=True, quant_input=qin)
+    sorted_ids, sorted_w, sorted_e, num_valid, _, sched = res[:6]
     ev = _mark("sort", ev)
     n_blk = sorted_e.numel()
     stream = _lib.current_stream()
@@ -204,12 +208,11 @@ def fused_moe(
                              num_valid_ids=num_valid, a2=a2, out3=out3, block_m=bm)
         return out
 
-    a1_q, a1_s = act_quant_mxfp4(hidden_states if hidden_states.stride(1) == 1 else hidden_states.contiguous())
+    a1_q, a1_s = res[6]
     # the stage-1 kernel writes its result already quantised for stage 2; the bf16 copy is only produced on request
     a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev) if return_parts else None
     a2_q = torch.empty(n_blk * bm, I // 2, dtype=torch.uint8, device=dev)
     a2_s = torch.empty(n_blk * bm, lib.pyhip_moe_act_scale_stride(I), dtype=torch.uint8, device=dev)
-    ev = _mark("quant1", ev)
     rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                    _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
                                    _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),

@@ -66,3 +66,29 @@ def test_sort_all_tokens_one_expert():
     T, k, E, Bm = 1000, 1, 8, 64
     ids = np.full((T, k), 5, dtype=np.int32)
     _run(ids, np.linspace(0, 1, T * k, dtype=np.float32).reshape(T, k), E, Bm)
+
+
+@pytest.mark.parametrize("T,k,E,Bm,K", [(16, 8, 256, 16, 7168), (200, 8, 64, 32, 1024), (256, 8, 256, 64, 2880 + 192),
+                                        (257, 8, 256, 64, 512), (3000, 4, 128, 128, 4096), (1, 1, 8, 16, 32)])
+def test_sort_with_quantisation_equals_the_separate_calls(T, k, E, Bm, K):
+    """pyhip_moe_sorting_quant carries the input quantisation in the sort's launches (the single-workgroup sort for
+    up to 2048 pairs, the scan launch above that): every output must equal the separate calls' bit for bit."""
+    from pyhip_amd.fused_moe import act_quant_mxfp4
+    rng = np.random.default_rng(T + K)
+    ids, w = _ids(rng, T, k, E, True), rng.random((T, k), dtype=np.float32)
+    dev = torch.device("cuda")
+    t_ids, t_w = torch.from_numpy(ids).to(dev), torch.from_numpy(w).to(dev)
+    x_full = (torch.randn(T, K + 64, generator=torch.Generator().manual_seed(T)) * 3).to(torch.bfloat16).to(dev)
+    x = x_full[:, :K]                                   # row stride larger than K
+    print(f"sort+quant case T={T} k={k} E={E} Bm={Bm} K={K}", flush=True)
+    ref = moe_sorting(t_ids, t_w, E, 64, torch.bfloat16, Bm, alloc_moe_out=False, return_schedule=True)
+    q_ref, s_ref = act_quant_mxfp4(x)
+    got = moe_sorting(t_ids, t_w, E, 64, torch.bfloat16, Bm, alloc_moe_out=False, return_schedule=True, quant_input=x)
+    torch.cuda.synchronize()
+    nv = int(ref[3][0])
+    assert torch.equal(got[3], ref[3])
+    assert torch.equal(got[0][:nv], ref[0][:nv]) and torch.equal(got[1][:nv], ref[1][:nv])
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1]) and torch.equal(got[2], ref[2])
+    assert torch.equal(got[5], ref[5])
+    q, s = got[6]
+    assert torch.equal(q, q_ref) and torch.equal(s, s_ref)
