@@ -31,7 +31,7 @@ PEAK_HBM_GBPS = 8000.0
 # FETCH_SIZE (x 2.0: a plain 1 GiB device copy reads 524 288) + WRITE_SIZE (x 1.0), KiB per dispatch,
 # collected with `rocprofv3 --pmc` around this script; other workloads report null.
 MEASURED_TRAFFIC = {
-    ("dsv3", 8192): 3.187e6 * 2 * 1024 + 1.018e5 * 1024,
+    ("dsv3", 8192): 3.252e6 * 2 * 1024 + 1.014e5 * 1024,
     ("dsv3", 16): 8.012e5 * 2 * 1024 + 6.765e3 * 1024,
 }
 
