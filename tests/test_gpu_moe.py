@@ -361,3 +361,45 @@ def test_graph_capture_replays(name, T, method):
         eager = fused_moe(hidden, w1, w2, tw, ti, **kw)  # eager work between the replays
         torch.cuda.synchronize()
         assert torch.equal(got, eager), f"replay {rep}"
+
+
+@pytest.mark.parametrize("method,T", [("a4w4", 200), ("w4a16", 6)])
+def test_expert_mask_and_local_tokens(method, T):
+    """Expert-parallel use of the call surface (src/contrib/fused_moe.py:134): with ``expert_mask`` a rank holds
+    the weights of its experts only and the sort hands out local expert ids; slots routed elsewhere contribute
+    nothing.  Every (token, slot) a rank owns must come out bit for bit as in the run that holds all experts,
+    and the ranks' fp32 outputs must add up to the full output.  ``num_local_tokens`` (a device scalar) limits
+    the tokens that take part without changing any launch shape."""
+    L = cases.make_layer("dsv3_s", T, seed=5)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    hidden = L.hidden.cuda()
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    E, N1, I = L.E, w1.shape[1], L.I
+    print(f"expert-mask case dsv3_s T={T} method={method}", flush=True)
+    full, pf = fused_moe(hidden, w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, dtype=torch.float32,
+                         return_parts=True, method=method, block_size_M=16)
+    total = torch.zeros_like(full)
+    # scale rows are grouped per expert: [E * N, ...] with N a multiple of 32, so an expert's rows can be selected
+    s1 = w1s.view(E, -1)
+    s2 = w2s.view(E, -1)
+    for parity in (0, 1):
+        mask = torch.tensor([(e % 2) == parity for e in range(E)], dtype=torch.int32, device="cuda")
+        keep = mask.bool()
+        out, p = fused_moe(hidden, w1[keep].contiguous(), w2[keep].contiguous(), tw, ti, expert_mask=mask,
+                           w1_scale=s1[keep].contiguous().view(-1, w1s.shape[-1]),
+                           w2_scale=s2[keep].contiguous().view(-1, w2s.shape[-1]),
+                           dtype=torch.float32, return_parts=True, method=method, block_size_M=16)
+        torch.cuda.synchronize()
+        mine = keep[ti.long()]                                   # [T, k]
+        assert torch.equal(p["out3"][mine], pf["out3"][mine])
+        assert (p["out3"][~mine] == 0).all()
+        total += out
+    assert torch.allclose(total, full, rtol=1e-5, atol=1e-6)
+
+    n_local = T // 2 + 1
+    nl = torch.tensor([n_local], dtype=torch.int32, device="cuda")
+    out = fused_moe(hidden, w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, dtype=torch.float32, num_local_tokens=nl,
+                    method=method, block_size_M=16)
+    torch.cuda.synchronize()
+    assert torch.equal(out[:n_local], full[:n_local])
+    assert (out[n_local:] == 0).all()
