@@ -403,3 +403,21 @@ def test_expert_mask_and_local_tokens(method, T):
     torch.cuda.synchronize()
     assert torch.equal(out[:n_local], full[:n_local])
     assert (out[n_local:] == 0).all()
+
+
+@pytest.mark.parametrize("method", ["a4w4", "w4a16"])
+def test_strided_hidden_states(method):
+    """hidden_states may be a column slice of a wider tensor (row stride larger than the hidden size): the result
+    is that of the contiguous copy, bit for bit"""
+    L = cases.make_layer("tiny", 40, seed=9)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    wide = torch.zeros(40, L.H + 256, dtype=torch.bfloat16, device="cuda")
+    wide[:, :L.H] = L.hidden.cuda()
+    view = wide[:, :L.H]
+    assert not view.is_contiguous()
+    print(f"strided hidden case method={method}", flush=True)
+    a = fused_moe(view, w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+    b = fused_moe(view.contiguous(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
