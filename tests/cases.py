@@ -15,6 +15,9 @@ CONFIGS = {
     # gpt-oss-shaped, scaled down: hidden = inter = 2880/2, not multiples of the kernels' 512-wide K tiles
     "gptoss_s": dict(E=16, k=4, H=1440, I=1440, router="softmax"),
     "gptoss_s1": dict(E=16, k=4, H=1536, I=1536, router="softmax"),         # 12 K-steps: an odd share per wave under split K
+    # an expert count that is not a multiple of the 8 XCDs the tile schedule deals experts to, an odd top-k,
+    # three K-groups in the gate_up GEMM
+    "odd": dict(E=12, k=3, H=1536, I=1024, router="softmax"),
 }
 
 

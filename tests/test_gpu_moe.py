@@ -126,6 +126,8 @@ def _end_to_end(got32, ref, ref_given_a2):
     ("qwen3_s", 257, 64, False),
     ("dsv3_s", 16, 16, False),
     ("dsv3_s", 128, None, False),
+    ("odd", 77, 32, True),
+    ("odd", 500, None, False),
 ])
 def test_fused_moe_matches_oracle(name, T, bm, bias):
     L = cases.make_layer(name, T, seed=0, bias=bias)
@@ -206,6 +208,7 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     ("qwen3_s", 64, 16, False, 1), ("dsv3_s", 16, None, False, 1), ("dsv3_s", 128, None, True, 1),
     ("tiny", 64, 16, True, 4), ("tiny", 200, 64, False, 4), ("mixtral_s", 33, 32, False, 4), ("dsv3_s", 16, None, False, 4),
     ("gptoss_s1", 20, 16, True, 4),
+    ("odd", 9, 16, False, 0), ("odd", 77, 32, True, 1),
 ])
 def test_w4a16_matches_oracle(name, T, bm, bias, splitk):
     """bf16 activations x MXFP4 weights (method="w4a16") against the oracle's "a16" path:
