@@ -46,6 +46,13 @@ def test_argument_errors_are_reported():
     one = ctypes.c_void_p(16)
     rc = lib.pyhip_moe_act_quant_mxfp4(one, 40, 4, 40, one, one, None, None)
     assert rc == 1 and b"multiple of 32" in lib.pyhip_moe_last_error()
+    # the sort that carries the input quantisation checks the quantiser's arguments before anything is launched
+    rc = lib.pyhip_moe_sorting_quant(one, one, 4, 2, 8, 16, None, None, one, one, one, one, None, one, 256,
+                                     one, 1024, 4, 1000, one, one, None)
+    assert rc == 1 and b"multiple of 32" in lib.pyhip_moe_last_error()
+    rc = lib.pyhip_moe_sorting_quant(one, one, 4, 2, 8, 16, None, None, one, one, one, one, None, one, 256,
+                                     None, 1024, 4, 1024, one, one, None)
+    assert rc == 1 and b"null pointer" in lib.pyhip_moe_last_error()
     rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1000, 512, 16, 4, 0, 0.0, None)
     assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
     rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 48, 4, None)
