@@ -165,6 +165,32 @@ int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t*
 int pyhip_moe_topk_reduce(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden, int out_is_f32,
                           const uint32_t* num_valid_ids, pyhip_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Zero fill of device memory with a kernel (safe inside a captured graph, where memset nodes are not).  The
+ * reference zeroes its buffers with torch (src/contrib/fused_moe.py:306, moe_sorting's moe_buf). */
+int pyhip_moe_zero_fill(void* p, int64_t bytes, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * The whole layer in one call: sort (+ input quantisation) -> gate_up GEMM -> down GEMM -> top-k reduce, i.e. the
+ * body of the reference's fused_moe (src/contrib/fused_moe.py:128-576) for the MXFP4 path, with every
+ * intermediate buffer carved out of `workspace` (pyhip_moe_forward_workspace_bytes() bytes, 256-byte aligned)
+ * instead of being allocated per call.  Enqueues on `stream`, never synchronises, allocates nothing.
+ *   hidden        bf16 [tokens, hidden], row stride hidden_row_stride elements (== hidden when w4a16 != 0)
+ *   w1, w2, scales, biases, expert_mask, num_local_tokens: as for the step-by-step entry points above
+ *   out           bf16 (or fp32 when out_is_f32 != 0) [tokens, hidden]
+ *   experts       the expert count the router saw (the length of expert_mask when one is given)
+ *   block_m       the row block: 16/32/64, with MXFP4 activations also 128/256
+ *   w4a16         0 = MXFP4 activations (pyhip_moe_gemm*_mxfp4), 1 = bf16 activations (pyhip_moe_gemm*_w4a16)
+ * pyhip_amd/fused_moe.py picks block_m and w4a16 (pick_block_m, pick_w4a16) and calls this. */
+int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                          int w4a16);
+int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1, const uint8_t* w1_scale,
+                      const uint8_t* w2, const uint8_t* w2_scale, const void* bias1_bf16, const void* bias2_bf16,
+                      const int32_t* topk_ids, const float* topk_weights, const int32_t* expert_mask,
+                      const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk, int experts,
+                      int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
+                      void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,150 @@
+// The whole layer behind one call: sort (+ input quantisation) -> gate_up GEMM -> down GEMM -> top-k reduce, with
+// every intermediate buffer carved out of a workspace the caller provides.  It is what pyhip_amd/fused_moe.py does
+// step by step (the reference's operator, src/contrib/fused_moe.py:128-576, allocates its intermediates with torch
+// and launches its kernels one by one from Python); the choice of kernel family and row block stays with the caller.
+#include "common.h"
+
+extern "C" {
+int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size);
+int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, int experts);
+int64_t pyhip_moe_schedule_words(int experts);
+int64_t pyhip_moe_act_scale_stride(int K);
+int pyhip_moe_sorting(const int32_t*, const float*, int, int, int, int, const int32_t*, const int32_t*, uint32_t*, float*,
+                      uint32_t*, uint32_t*, uint32_t*, void*, int64_t, void*, int64_t, hipStream_t);
+int pyhip_moe_sorting_quant(const int32_t*, const float*, int, int, int, int, const int32_t*, const int32_t*, uint32_t*,
+                            float*, uint32_t*, uint32_t*, uint32_t*, void*, int64_t, const void*, int64_t, int64_t, int,
+                            uint8_t*, uint8_t*, hipStream_t);
+int pyhip_moe_gemm1_mxfp4(const uint8_t*, const uint8_t*, const uint8_t*, const uint8_t*, const void*, const uint32_t*,
+                          const uint32_t*, const uint32_t*, const uint32_t*, void*, uint8_t*, uint8_t*, int, int, int, int,
+                          int, int, int64_t, int, float, hipStream_t);
+int pyhip_moe_gemm2_mxfp4(const uint8_t*, const uint8_t*, const uint8_t*, const uint8_t*, const void*, const uint32_t*,
+                          const float*, const uint32_t*, const uint32_t*, const uint32_t*, void*, int, int, int, int, int,
+                          int, int64_t, hipStream_t);
+int pyhip_moe_gemm1_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const uint32_t*,
+                          const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, int, float, hipStream_t);
+int pyhip_moe_gemm2_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const float*,
+                          const uint32_t*, const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, hipStream_t);
+int pyhip_moe_topk_reduce(const void*, void*, int64_t, int, int, int, const uint32_t*, hipStream_t);
+int pyhip_moe_zero_fill(void* p, int64_t bytes, hipStream_t stream);
+}
+
+namespace {
+struct Carve
+{
+    int64_t off = 0;
+    int64_t take(int64_t bytes)
+    {
+        int64_t o = off;
+        off += (bytes + 255) / 256 * 256;
+        return o;
+    }
+};
+struct Layout
+{
+    int64_t n_blk, rows2;
+    int64_t sorted_ids, sorted_w, sorted_e, num_valid, sched, sort_ws, sort_ws_bytes, a1_q, a1_s, a2, a2_q, a2_s, out3;
+    int64_t total;
+};
+Layout make_layout(int64_t T, int k, int E, int H, int I, int bm, int w4a16)
+{
+    Layout l;
+    Carve c;
+    l.n_blk         = pyhip_moe_sorting_max_blocks(T, k, E, bm);
+    l.rows2         = l.n_blk * bm;
+    l.sorted_ids    = c.take(l.rows2 * 4);
+    l.sorted_w      = c.take(l.rows2 * 4);
+    l.sorted_e      = c.take(l.n_blk * 4);
+    l.num_valid     = c.take(8);
+    l.sched         = c.take(pyhip_moe_schedule_words(E) * 4);
+    l.sort_ws_bytes = pyhip_moe_sorting_workspace_bytes(T, k, E);
+    l.sort_ws       = c.take(l.sort_ws_bytes);
+    l.a1_q = l.a1_s = l.a2 = l.a2_q = l.a2_s = 0;
+    if(w4a16)
+        l.a2 = c.take(l.rows2 * (int64_t)I * 2);
+    else
+    {
+        l.a1_q = c.take(T * (int64_t)(H / 2));
+        l.a1_s = c.take(T * pyhip_moe_act_scale_stride(H));
+        l.a2_q = c.take(l.rows2 * (int64_t)(I / 2));
+        l.a2_s = c.take(l.rows2 * pyhip_moe_act_scale_stride(I));
+    }
+    l.out3  = c.take(T * (int64_t)k * H * 2);
+    l.total = c.off;
+    return l;
+}
+}   // namespace
+
+extern "C" int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, int experts, int hidden, int inter,
+                                                     int block_m, int w4a16)
+{
+    if(tokens <= 0 || topk <= 0 || experts <= 0 || hidden <= 0 || inter <= 0 || block_m <= 0)
+        return 0;
+    return make_layout(tokens, topk, experts, hidden, inter, block_m, w4a16).total;
+}
+
+extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
+                                 const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                                 const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
+                                 const float* topk_weights, const int32_t* expert_mask,
+                                 const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk,
+                                 int experts, int hidden, int inter, int block_m, int w4a16, int split_k,
+                                 int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
+                                 hipStream_t stream)
+{
+    PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && w2 && w2_scale && topk_ids && topk_weights && out,
+                  "moe_forward: null pointer");
+    PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0 && hidden > 0 && inter > 0, "moe_forward: bad sizes");
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || ((block_m == 128 || block_m == 256) && !w4a16),
+                  "moe_forward: block_m=%d (16/32/64, and 128/256 with MXFP4 activations)", block_m);
+    PYHIP_REQUIRE(!w4a16 || hidden_row_stride == hidden, "moe_forward: the bf16-activation kernels need contiguous rows");
+    const Layout l = make_layout(tokens, topk, experts, hidden, inter, block_m, w4a16);
+    PYHIP_REQUIRE(workspace && workspace_bytes >= l.total && ((uintptr_t)workspace % 256) == 0,
+                  "moe_forward: workspace of %lld bytes (256-byte aligned) needed, %lld given", (long long)l.total,
+                  (long long)workspace_bytes);
+    uint8_t* ws       = (uint8_t*)workspace;
+    uint32_t* s_ids   = (uint32_t*)(ws + l.sorted_ids);
+    float* s_w        = (float*)(ws + l.sorted_w);
+    uint32_t* s_e     = (uint32_t*)(ws + l.sorted_e);
+    uint32_t* n_valid = (uint32_t*)(ws + l.num_valid);
+    uint32_t* sched   = (uint32_t*)(ws + l.sched);
+    void* out3        = ws + l.out3;
+    int rc;
+    if(w4a16)
+        rc = pyhip_moe_sorting(topk_ids, topk_weights, tokens, topk, experts, block_m, expert_mask, num_local_tokens,
+                               s_ids, s_w, s_e, n_valid, sched, nullptr, 0, ws + l.sort_ws, l.sort_ws_bytes, stream);
+    else
+        rc = pyhip_moe_sorting_quant(topk_ids, topk_weights, tokens, topk, experts, block_m, expert_mask,
+                                     num_local_tokens, s_ids, s_w, s_e, n_valid, sched, ws + l.sort_ws, l.sort_ws_bytes,
+                                     hidden_bf16, hidden_row_stride, tokens, hidden, ws + l.a1_q, ws + l.a1_s, stream);
+    if(rc)
+        return rc;
+    // slots routed to experts this rank does not hold, and tokens past the local count, contribute nothing
+    if(expert_mask || num_local_tokens)
+    {
+        rc = pyhip_moe_zero_fill(out3, (int64_t)tokens * topk * hidden * 2, stream);
+        if(rc)
+            return rc;
+    }
+    if(w4a16)
+    {
+        rc = pyhip_moe_gemm1_w4a16(hidden_bf16, w1, w1_scale, bias1_bf16, s_ids, s_e, n_valid, ws + l.a2, tokens, topk,
+                                   experts, hidden, inter, block_m, l.n_blk, split_k, activation, swiglu_limit, stream);
+        if(rc)
+            return rc;
+        rc = pyhip_moe_gemm2_w4a16(ws + l.a2, w2, w2_scale, bias2_bf16, s_ids, s_w, s_e, n_valid, out3, tokens, topk,
+                                   experts, hidden, inter, block_m, l.n_blk, split_k, stream);
+    }
+    else
+    {
+        rc = pyhip_moe_gemm1_mxfp4(ws + l.a1_q, ws + l.a1_s, w1, w1_scale, bias1_bf16, s_ids, s_e, n_valid, sched, nullptr,
+                                   ws + l.a2_q, ws + l.a2_s, tokens, topk, experts, hidden, inter, block_m, l.n_blk,
+                                   activation, swiglu_limit, stream);
+        if(rc)
+            return rc;
+        rc = pyhip_moe_gemm2_mxfp4(ws + l.a2_q, ws + l.a2_s, w2, w2_scale, bias2_bf16, s_ids, s_w, s_e, n_valid, sched,
+                                   out3, tokens, topk, experts, hidden, inter, block_m, l.n_blk, stream);
+    }
+    if(rc)
+        return rc;
+    return pyhip_moe_topk_reduce(out3, out, tokens, topk, hidden, out_is_f32, nullptr, stream);
+}

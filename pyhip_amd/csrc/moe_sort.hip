@@ -479,6 +479,23 @@ extern "C" __global__ void moe_zero_kernel(uint4* p, size_t n16, unsigned char* 
         tail[threadIdx.x] = 0;
 }
 
+// zero fill of `bytes` bytes of device memory with a kernel (a memset node does not replay reliably inside a
+// captured graph); used for buffers that only some rows are written to
+extern "C" int pyhip_moe_zero_fill(void* p, int64_t bytes, hipStream_t stream)
+{
+    PYHIP_REQUIRE(p && bytes >= 0 && ((uintptr_t)p % 16) == 0, "zero_fill: bad buffer");
+    if(bytes == 0)
+        return PYHIP_OK;
+    size_t n16 = (size_t)bytes / 16;
+    int ntail  = (int)(bytes - (int64_t)n16 * 16);
+    int grid   = (int)((n16 + 255) / 256);
+    grid       = grid < 1 ? 1 : (grid > 2048 ? 2048 : grid);
+    hipLaunchKernelGGL(moe_zero_kernel, dim3(grid), dim3(256), 0, stream, (uint4*)p, n16, (unsigned char*)p + n16 * 16,
+                       ntail);
+    PYHIP_CHECK_LAUNCH("moe_zero_kernel");
+    return PYHIP_OK;
+}
+
 // ---------------------------------------------------------------------------------------------
 #define SMALL_PAIRS_MAX (SMALL_WAVES * SMALL_GROUPS * WAVE)
 #define MAX_EXPERTS 2048

@@ -161,6 +161,36 @@ def fused_moe(
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E, H)
     if w4a16:
         bm = min(bm, 64)
+    if bias1 is not None:
+        bias1 = bias1.to(torch.bfloat16).contiguous()
+        assert tuple(bias1.shape) == (E, 2 * I)
+    if bias2 is not None:
+        bias2 = bias2.to(torch.bfloat16).contiguous()
+        assert tuple(bias2.shape) == (E, H)
+
+    if not return_parts and stage_events is None:
+        # the whole layer in one library call, intermediates in one workspace: two allocations and one foreign call
+        # per layer instead of a dozen of each (the host side is what bounds small layers when they are not replayed
+        # from a graph)
+        if expert_mask is not None:
+            expert_mask = expert_mask.to(device=dev, dtype=torch.int32).contiguous()
+        if num_local_tokens is not None:
+            assert num_local_tokens.is_cuda and num_local_tokens.dtype == torch.int32
+        x = hidden_states
+        if x.stride(1) != 1 or (w4a16 and x.stride(0) != H):
+            x = x.contiguous()
+        ws_bytes = lib.pyhip_moe_forward_workspace_bytes(T, k, global_E, H, I, bm, 1 if w4a16 else 0)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        out = torch.empty(T, H, dtype=out_dtype, device=dev)
+        rc = lib.pyhip_moe_forward(_lib.dptr(x), x.stride(0), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(w2u),
+                                   _lib.dptr(w2s), _lib.dptr(bias1), _lib.dptr(bias2), _lib.dptr(topk_ids),
+                                   _lib.dptr(topk_weight), _lib.dptr(expert_mask), _lib.dptr(num_local_tokens),
+                                   _lib.dptr(out), 1 if out_dtype == torch.float32 else 0, T, k, global_E, H, I, bm,
+                                   1 if w4a16 else 0, splitk, act, limit, _lib.dptr(ws), ws_bytes,
+                                   _lib.current_stream())
+        _lib.check(rc, "moe_forward")
+        return out[:, : H - hidden_pad] if narrow else out
+
     ev = _mark("start")
     # MXFP4-activation path: the input quantisation rides in the sort's launches (independent work, one dispatch less)
     qin = None
@@ -172,13 +202,6 @@ def fused_moe(
     ev = _mark("sort", ev)
     n_blk = sorted_e.numel()
     stream = _lib.current_stream()
-
-    if bias1 is not None:
-        bias1 = bias1.to(torch.bfloat16).contiguous()
-        assert tuple(bias1.shape) == (E, 2 * I)
-    if bias2 is not None:
-        bias2 = bias2.to(torch.bfloat16).contiguous()
-        assert tuple(bias2.shape) == (E, H)
 
     if w4a16:
         hs = hidden_states.contiguous()

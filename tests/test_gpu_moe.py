@@ -424,3 +424,29 @@ def test_strided_hidden_states(method):
     b = fused_moe(view.contiguous(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("name,T,method,bias", [("tiny", 64, "a4w4", True), ("tiny", 5, "w4a16", True),
+                                                ("dsv3_s", 300, "a4w4", False), ("odd", 40, "auto", False)])
+def test_one_call_path_equals_the_step_by_step_path(name, T, method, bias):
+    """Without ``return_parts`` / ``stage_events`` the operator is a single pyhip_moe_forward call with one workspace;
+    with them it runs the entry points one by one with separate buffers.  Same kernels, same order: same bits, with
+    and without an expert mask and a local token count."""
+    L = cases.make_layer(name, T, seed=12, bias=bias)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    b1 = None if L.bias1 is None else L.bias1.cuda()
+    b2 = None if L.bias2 is None else L.bias2.cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s, bias1=b1, bias2=b2, method=method)
+    print(f"one-call case {name} T={T} method={method} bias={bias}", flush=True)
+    hidden = L.hidden.cuda()
+    for dt in (None, torch.float32):
+        a = fused_moe(hidden, w1, w2, tw, ti, dtype=dt, **kw)
+        b, _ = fused_moe(hidden, w1, w2, tw, ti, dtype=dt, return_parts=True, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
+    nl = torch.tensor([T // 2], dtype=torch.int32, device="cuda")
+    a = fused_moe(hidden, w1, w2, tw, ti, num_local_tokens=nl, **kw)
+    b, _ = fused_moe(hidden, w1, w2, tw, ti, num_local_tokens=nl, return_parts=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and (a[T // 2:] == 0).all()
