@@ -74,6 +74,25 @@ Layout make_layout(int64_t T, int k, int E, int H, int I, int bm, int w4a16)
 }
 }   // namespace
 
+// The choices pyhip_amd/fused_moe.py makes for method="auto" and block_size_M=None (pick_block_m, pick_w4a16; the
+// measurements behind them are quoted there), for callers that bind the library without the Python layer.
+extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int hidden)
+{
+    const double est = (double)tokens * topk / (experts > 0 ? experts : 1);      // routed rows per expert, on average
+    for(int bm = 16; bm <= 64; bm *= 2)
+        if(2 * est <= bm)
+            return bm;
+    return (hidden >= 6144 && est >= 120 && est <= 192) ? 256 : 128;
+}
+
+extern "C" int pyhip_moe_pick_w4a16(int64_t tokens, int topk, int experts, int hidden)
+{
+    const int64_t pairs  = tokens * topk;
+    const bool sparse    = 4 * pairs <= 3 * (int64_t)experts;
+    const bool few_tiles = (pairs < experts ? pairs : experts) * (hidden / 256) < 512 && pairs <= 8 * (int64_t)experts;
+    return sparse || few_tiles;
+}
+
 extern "C" int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, int experts, int hidden, int inter,
                                                      int block_m, int w4a16)
 {

@@ -100,3 +100,14 @@ def test_auto_method_rule():
     assert pick_w4a16(1, 2, 8, 4096) and pick_w4a16(32, 2, 8, 4096)               # Mixtral: 8 experts x 16 tiles
     assert not pick_w4a16(48, 2, 8, 4096) and not pick_w4a16(4096, 2, 8, 4096)
     assert not pick_w4a16(64, 2, 8, 1024)                                         # the tiny shape at 16 rows per expert
+
+
+def test_library_makes_the_same_choices():
+    """pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 (for callers without the Python layer) agree with the host code"""
+    from pyhip_amd import _lib
+    from pyhip_amd.fused_moe import pick_block_m, pick_w4a16
+    lib = _lib.load()
+    for E, k, H in ((8, 2, 1024), (8, 2, 4096), (128, 4, 3072), (128, 8, 4096), (256, 8, 7168), (12, 3, 1536)):
+        for T in list(range(1, 70)) + [96, 128, 200, 256, 500, 512, 1000, 1024, 2048, 3072, 3840, 4096, 5000, 6144, 6145, 8192, 32768]:
+            assert lib.pyhip_moe_pick_block_m(T, k, E, H) == pick_block_m(T, k, E, H), (T, k, E, H)
+            assert bool(lib.pyhip_moe_pick_w4a16(T, k, E, H)) == pick_w4a16(T, k, E, H), (T, k, E, H)
