@@ -112,9 +112,13 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     constexpr int KSTRIDE = SPLITK ? 4 : 1;
     v4i wf[2][4];
     v4i af[2][MT][4];
-    u32 wsc[4];                // scale dwords of the current 256-K column tile (two K-steps)
+    u32 wsc[2][4];             // scale dwords (one covers the two K-steps of a 256-K column tile), loaded with
+                               // the K-step's weights: fetched only when needed, their latency would add to every step
     auto load_step = [&](auto BB, int kt) __attribute__((always_inline)) {
         constexpr int buf = decltype(BB)::value;
+#pragma unroll
+        for(int j = 0; j < 4; j++)
+            wsc[buf][j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
 #pragma unroll
         for(int j = 0; j < 4; j++)
             wf[buf][j] = __builtin_nontemporal_load((const v4i*)(wp[j] + (size_t)kt * 1024));
@@ -127,12 +131,6 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     // one K-step from register set P while the next one loads into set 1 - P (K / 128 is even)
     auto k_step = [&](auto PP, int kt) __attribute__((always_inline)) {
         constexpr int P = decltype(PP)::value;
-        if(P == 0 || SPLITK)
-        {
-#pragma unroll
-            for(int j = 0; j < 4; j++)
-                wsc[j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
-        }
         if(kt + KSTRIDE < KT)
             load_step(std::integral_constant<int, 1 - P>{}, kt + KSTRIDE);
 #pragma unroll
@@ -140,7 +138,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
         {
             // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
             const int kpar = SPLITK ? (kt & 1) : P;          // without the split the parity is the register set
-            const u32 sb   = (wsc[j] >> (8 * (kpar * 2 + sbyte_row[j]))) & 0xFFu;
+            const u32 sb   = (wsc[P][j] >> (8 * (kpar * 2 + sbyte_row[j]))) & 0xFFu;
             v8bf wq[4];
             expand_fp4(wf[P][j], sb, wq);
 #pragma unroll
