@@ -4,20 +4,24 @@
 A step is one ``fused_moe`` call (sort -> quantise -> gate_up GEMM -> quantise -> down GEMM -> top-k
 reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
 
-  value     TFLOP/s of the whole layer at --tokens (default 8192), FLOPs = 6*T*k*I*H
-  decode    the same layer at --decode-tokens (default 16): ms, HBM GB/s on algorithmic bytes (method="auto":
-            bf16 activations x MXFP4 weights at this size)
-            bf16 activations x MXFP4 weights at this size); graph_replay_ms_per_step is the same call captured in
-            a HIP graph and replayed
-  decode_a4w4  the same with MXFP4 activations forced (method="a4w4")
-  sweep     the same layer at --sweep-tokens (default 128, 1024, 4096): ms, TFLOP/s and GB/s on algorithmic work
-  roofline  the dominant kernel (stage-1 gate_up GEMM) of the primary workload, timed with events
-            recorded around it inside the timed steps (every fourth one)
-  cpu_baseline  the CPU oracle (oracle/moe.py) on a bounded sample of the same workload
+  value        TFLOP/s of the whole layer at the headline workload (DeepSeek-V3 shape, 8192 tokens),
+               FLOPs = 6*T*k*I*H, wall clock over exactly --steps calls of the one-call product path
+  configs      every benchmark point (five shapes x their token counts): method and row block the operator
+               picked, median and inter-quartile range of the time per call (HIP events around batches of
+               back-to-back calls, product path only), TFLOP/s and GB/s on the algorithmic work and both
+               roofline fractions.  Layers whose weights fit the 256 MB last-level cache rotate over
+               several copies of the weights, as the reference's harness does (src/misc.py:180-273)
+  decode       the headline shape at --decode-tokens (default 16), the HBM-bound end of the metric, with the
+               same call captured in a HIP graph and replayed
+  roofline     the dominant kernel (stage-1 gate_up GEMM) of the headline workload: average launch duration
+               from HIP events recorded on the launch stream around that launch in a separate, untimed pass
+               of the step-by-step path; traffic is read from the committed counter summary under profiles/
+  cpu_baseline the CPU oracle (oracle/moe.py) on a bounded sample of the headline workload
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,14 +30,17 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_FP4_TFLOPS = 10100.0     # MI355X dense MXFP4/MXFP6
 PEAK_HBM_GBPS = 8000.0
+LAST_LEVEL_CACHE_BYTES = 256 << 20
 
-# HBM-side bytes per launch of the gate_up GEMM, (shape, tokens) -> bytes, from the hardware counters
-# FETCH_SIZE (x 2.0: a plain 1 GiB device copy reads 524 288) + WRITE_SIZE (x 1.0), KiB per dispatch,
-# collected with `rocprofv3 --pmc` around this script; other workloads report null.
-MEASURED_TRAFFIC = {
-    ("dsv3", 8192): 3.252e6 * 2 * 1024 + 1.014e5 * 1024,
-    ("dsv3", 16): 8.012e5 * 2 * 1024 + 6.765e3 * 1024,
+# the benchmark points: shape -> token counts
+POINTS = {
+    "tiny": [64],
+    "mixtral": [1, 32, 512, 4096],
+    "gptoss": [16, 256, 4096],
+    "qwen3": [64, 2048, 8192],
+    "dsv3": [16, 128, 1024, 8192],
 }
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "fused_moe_dsv3_hbm_traffic.txt")
 
 
 def parse():
@@ -41,65 +48,138 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--shape", default="dsv3")
+    ap.add_argument("--shape", default="dsv3", help="shape of the headline workload")
     ap.add_argument("--tokens", type=int, default=8192)
     ap.add_argument("--decode-tokens", type=int, default=16)
-    ap.add_argument("--sweep-tokens", type=lambda v: [int(x) for x in v.split(",") if x], default=[128, 1024, 4096],
-                    help="further token counts reported in 'sweep' (comma separated; empty = none)")
+    ap.add_argument("--points", default="all",
+                    help="'all', 'none', or a comma separated list like dsv3:16,qwen3:8192 for the 'configs' array")
     ap.add_argument("--block-m", type=int, default=0)
+    ap.add_argument("--method", default="auto")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="target size of the CPU sample; 0 = skip")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
     return ap.parse_args()
 
 
-def run_config(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, method="auto"):
+def call_kwargs(W, block_m, method):
+    return dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
+                block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"],
+                method=method)
+
+
+def weight_copies(torch, W, work):
+    """the weights the timed calls rotate over: one set when a call's working set exceeds the last-level cache
+    twice over, otherwise enough copies that consecutive calls cannot find their weights cached"""
+    if work["bytes"] >= 2 * LAST_LEVEL_CACHE_BYTES:
+        return [W]
+    total = sum(W[k].numel() * W[k].element_size() for k in ("w1", "w2", "w1_scale", "w2_scale"))
+    n = int(min(64, max(2, -(-(3 * LAST_LEVEL_CACHE_BYTES) // max(work["bytes"], 1)))))
+    n = int(max(2, min(n, (4 << 30) // max(total, 1))))
+    copies = [W]
+    for _ in range(n - 1):
+        C = dict(W)
+        for k in ("w1", "w2", "w1_scale", "w2_scale"):
+            C[k] = W[k].clone()
+        C["w1"].is_shuffled = C["w2"].is_shuffled = True
+        copies.append(C)
+    return copies
+
+
+def time_point(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, method="auto"):
+    """-> dict with wall-clock ms over exactly `steps` calls, and median / IQR over event-timed batches; only the
+    one-call product path runs inside the timed regions"""
     from pyhip_amd import workloads
+    from pyhip_amd.fused_moe import pick_block_m, pick_w4a16
     hidden, topk_w, topk_ids = workloads.make_inputs(shape, tokens)
     if W["hidden_pad"]:      # padded shapes (gpt-oss): activations at the padded width, as the reference passes them
         hidden = torch.nn.functional.pad(hidden, (0, W["hidden_pad"]))
-    kw = dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
-              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"],
-              method=method)
-    for _ in range(warmup):
-        out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, **kw)
+    work = workloads.algorithmic_work(shape, tokens, topk_ids)
+    sets = weight_copies(torch, W, work)
+    kws = [call_kwargs(C, block_m, method) for C in sets]
+
+    def call(i):
+        C = sets[i % len(sets)]
+        return fused_moe(hidden, C["w1"], C["w2"], topk_w, topk_ids, **kws[i % len(sets)])
+
+    for i in range(max(warmup, len(sets))):
+        out = call(i)
     torch.cuda.synchronize()
-    events = []
     t0 = time.perf_counter()
     for i in range(steps):
-        # stage events on every fourth timed step: recording one costs several microseconds of GPU time
-        out = fused_moe(hidden, W["w1"], W["w2"], topk_w, topk_ids, stage_events=events if i % 4 == 0 else None, **kw)
+        out = call(i)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     assert torch.isfinite(out.float()).all()
-    stage_ms = {}
+    # event-timed batches: enough calls per batch that the events' own cost (microseconds) does not show
+    reps = int(max(1, min(64, round(2.0 / max(wall_ms, 1e-3)))))
+    batches = 15
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(batches + 1)]
+    evs[0].record()
+    n = 0
+    for b in range(batches):
+        for _ in range(reps):
+            call(n)
+            n += 1
+        evs[b + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(evs[b].elapsed_time(evs[b + 1]) / reps for b in range(batches))
+    q = lambda f: per[min(batches - 1, int(f * batches))]
+    cfg = workloads.SHAPES[shape]
+    Hp = cfg["H"] + W["hidden_pad"]
+    w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(tokens, cfg["k"], cfg["E"], Hp))
+    bm = block_m or pick_block_m(tokens, cfg["k"], cfg["E"], Hp)
+    return dict(wall_ms=wall_ms, median_ms=q(0.5), q1_ms=q(0.25), q3_ms=q(0.75), work=work, hidden=hidden,
+                topk_w=topk_w, topk_ids=topk_ids, out=out, method="w4a16" if w4a16 else "a4w4",
+                block_m=min(bm, 64) if w4a16 else bm, weight_copies=len(sets), calls_per_batch=reps)
+
+
+def stage_pass(torch, fused_moe, W, res, block_m, method, passes=8):
+    """average duration of each launch group of the step-by-step path, from events on the launch stream; untimed
+    (not part of any ms_per_step)"""
+    kw = call_kwargs(W, block_m, method)
+    events = []
+    for _ in range(2):
+        fused_moe(res["hidden"], W["w1"], W["w2"], res["topk_w"], res["topk_ids"], stage_events=[], **kw)
+    for _ in range(passes):
+        fused_moe(res["hidden"], W["w1"], W["w2"], res["topk_w"], res["topk_ids"], stage_events=events, **kw)
+    torch.cuda.synchronize()
+    acc = {}
     for name, a, b in events:
-        stage_ms.setdefault(name, []).append(a.elapsed_time(b))
-    stage_ms = {k: sum(v) / len(v) for k, v in stage_ms.items()}
-    work = workloads.algorithmic_work(shape, tokens, topk_ids)
-    return dict(ms=wall * 1e3 / steps, stage_ms=stage_ms, work=work, hidden=hidden, topk_w=topk_w, topk_ids=topk_ids,
-                out=out)
+        acc.setdefault(name, []).append(a.elapsed_time(b))
+    return {k: sum(v) / len(v) for k, v in acc.items()}
 
 
 def graph_replay_ms(torch, fused_moe, W, res, steps, block_m, method="auto"):
     """the same call captured once in a HIP graph and replayed: what a serving loop that captures its decode step
     pays per layer (no host work between the launches)"""
-    kw = dict(w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], bias1=W.get("bias1"), bias2=W.get("bias2"),
-              block_size_M=block_m or None, hidden_pad=W["hidden_pad"], intermediate_pad=W["intermediate_pad"],
-              method=method)
+    kw = call_kwargs(W, block_m, method)
     args = (res["hidden"], W["w1"], W["w2"], res["topk_w"], res["topk_ids"])
+    eager = fused_moe(*args, **kw)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out = fused_moe(*args, **kw)
     for _ in range(5):
         graph.replay()
     torch.cuda.synchronize()
-    assert torch.equal(out, res["out"]), "graph replay differs from the eager result"
+    assert torch.equal(out, eager), "graph replay differs from the eager result"
     t0 = time.perf_counter()
     for _ in range(steps):
         graph.replay()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def measured_traffic(kernel_key):
+    """HBM-side bytes per launch of a kernel from the committed counter summary (lines of the form
+    `traffic_bytes_per_launch <key> <bytes>`, written when the counters were collected, with the commit they
+    were collected at); None when the summary has no such line"""
+    try:
+        text = open(TRAFFIC_FILE).read()
+    except OSError:
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch\s+%s\s+([0-9.eE+]+)" % re.escape(kernel_key), text, re.M)
+    c = re.search(r"^collected_at\s+(.+)$", text, re.M)
+    return (float(m.group(1)) if m else None), (c.group(1).strip() if c else None)
 
 
 class LazyExperts:
@@ -149,6 +229,17 @@ def cpu_baseline(torch, W, shape, res, budget_s):
                        % (len(done), len(hit), pairs, ids.size, shape, ids.shape[0], t_total))
 
 
+def point_record(shape, tokens, r):
+    w, ms = r["work"], r["median_ms"]
+    tfl = w["flops"] / (ms * 1e-3) / 1e12
+    gbs = w["bytes"] / (ms * 1e-3) / 1e9
+    return {"shape": shape, "tokens": tokens, "method": r["method"], "block_m": r["block_m"], "experts_hit": w["e_hit"],
+            "ms_median": round(ms, 4), "ms_iqr": [round(r["q1_ms"], 4), round(r["q3_ms"], 4)],
+            "ms_wall_mean": round(r["wall_ms"], 4), "tflops": round(tfl, 1),
+            "frac_of_mfma_peak": round(tfl / PEAK_MFMA_FP4_TFLOPS, 4), "hbm_gbps": round(gbs, 1),
+            "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBPS, 4), "weight_copies": r["weight_copies"]}
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -158,23 +249,39 @@ def main():
     import torch
     from pyhip_amd import fused_moe, workloads
     torch.cuda.set_device(0)
+    if a.points == "all":
+        points = [(s, t) for s, ts in POINTS.items() for t in ts]
+    elif a.points in ("none", ""):
+        points = []
+    else:
+        points = [(p.split(":")[0], int(p.split(":")[1])) for p in a.points.split(",")]
+
     cfg = workloads.SHAPES[a.shape]
-    W = workloads.make_weights(a.shape)
-    torch.cuda.synchronize()
-    main_res = run_config(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m)
-    dec = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
-    dec4 = run_config(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
-    dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
-    # the same layer at sizes between the two headline points (method and row block chosen by the operator)
-    sweep = []
-    for t in a.sweep_tokens:
-        r = run_config(torch, fused_moe, W, a.shape, t, a.steps, a.warmup, a.block_m)
-        sweep.append({"tokens": t, "ms_per_step": round(r["ms"], 4),
-                      "tflops": round(r["work"]["flops"] / (r["ms"] * 1e-3) / 1e12, 1),
-                      "frac_of_mfma_peak": round(r["work"]["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_MFMA_FP4_TFLOPS, 4),
-                      "hbm_gbps": round(r["work"]["bytes"] / (r["ms"] * 1e-3) / 1e9, 1),
-                      "frac_of_hbm_peak": round(r["work"]["bytes"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)})
-        del r
+    configs = []
+    main_res = dec = None
+    shapes = list(dict.fromkeys([s for s, _ in points] + [a.shape]))
+    shapes.sort(key=lambda s: s == a.shape)              # the headline shape last: its results feed the rest of the line
+    for shape in shapes:
+        W = workloads.make_weights(shape)
+        torch.cuda.synchronize()
+        for s, t in points:
+            if s != shape:
+                continue
+            steps, warm = (a.steps, a.warmup) if t >= 1024 else (max(a.steps, 50), max(a.warmup, 10))
+            r = time_point(torch, fused_moe, W, s, t, steps, warm, 0, "auto")
+            configs.append(point_record(s, t, r))
+            del r
+        if shape == a.shape:
+            # headline: exactly --steps timed calls after --warmup untimed ones
+            main_res = time_point(torch, fused_moe, W, a.shape, a.tokens, a.steps, a.warmup, a.block_m, a.method)
+            main_stage = stage_pass(torch, fused_moe, W, main_res, a.block_m, a.method)
+            dec = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
+            dec_stage = stage_pass(torch, fused_moe, W, dec, a.block_m, "auto")
+            dec4 = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
+            dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
+            cpu = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds) if a.cpu_seconds > 0 else None
+        del W
+        torch.cuda.empty_cache()
 
     if a.calibrate_copy:
         src = torch.zeros(a.calibrate_copy << 20, dtype=torch.uint8, device="cuda")
@@ -185,48 +292,54 @@ def main():
         del src, dst
 
     w = main_res["work"]
-    tflops = w["flops"] / (main_res["ms"] * 1e-3) / 1e12
-    g1_ms = main_res["stage_ms"]["gemm1"]
+    tflops = w["flops"] / (main_res["wall_ms"] * 1e-3) / 1e12
+    g1_ms = main_stage["gemm1"]
     g1_tflops = w["flops_stage1"] / (g1_ms * 1e-3) / 1e12
     dw = dec["work"]
-    dec_gbps = dw["bytes"] / (dec["ms"] * 1e-3) / 1e9
-    dg1_ms = dec["stage_ms"]["gemm1"]
+    dec_gbps = dw["bytes"] / (dec["median_ms"] * 1e-3) / 1e9
+    dg1_ms = dec_stage["gemm1"]
+    traffic, collected = measured_traffic("gate_up_%s_T%d" % (a.shape, a.tokens))
+    dtraffic, _ = measured_traffic("gate_up_%s_T%d" % (a.shape, a.decode_tokens))
     out = {
         "metric": "MXFP4 fused-MoE TFLOP/s (DeepSeek-V3 routed-expert layer, %d tokens); decode-size HBM GB/s in 'decode'"
                   % a.tokens if a.shape == "dsv3" else "MXFP4 fused-MoE TFLOP/s (%s, %d tokens)" % (a.shape, a.tokens),
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(main_res["ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(main_res["wall_ms"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "mxfp4 (e2m1 x e2m1, e8m0 1x32 scales, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "%s E=%d top%d H=%d I=%d T=%d" % (a.shape, cfg["E"], cfg["k"], cfg["H"], cfg["I"], a.tokens),
-                   "experts_hit": w["e_hit"], "block_m": a.block_m or "auto"},
+                   "experts_hit": w["e_hit"], "method": main_res["method"], "block_m": main_res["block_m"]},
+        "ms_median": round(main_res["median_ms"], 4), "ms_iqr": [round(main_res["q1_ms"], 4), round(main_res["q3_ms"], 4)],
         "frac_of_mfma_peak": round(tflops / PEAK_MFMA_FP4_TFLOPS, 4),
-        "hbm_gbps": round(w["bytes"] / (main_res["ms"] * 1e-3) / 1e9, 1),
-        "stage_ms": {k: round(v, 4) for k, v in main_res["stage_ms"].items()},
+        "hbm_gbps": round(w["bytes"] / (main_res["wall_ms"] * 1e-3) / 1e9, 1),
+        "frac_of_hbm_peak": round(w["bytes"] / (main_res["wall_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+        "stage_ms_untimed_pass": {k: round(v, 4) for k, v in main_stage.items()},
         "roofline": {"kernel": "moe_gemm_mxfp4_kernel<1,*> (gate_up)", "bound": "mfma", "achieved": round(g1_tflops, 2),
                      "peak": PEAK_MFMA_FP4_TFLOPS, "unit": "TFLOP/s", "frac": round(g1_tflops / PEAK_MFMA_FP4_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get((a.shape, a.tokens)), "avg_launch_ms": round(g1_ms, 4),
+                     "traffic": traffic, "traffic_source": None if traffic is None else
+                     "profiles/%s (%s)" % (os.path.basename(TRAFFIC_FILE), collected or "commit not recorded"),
+                     "avg_launch_ms": round(g1_ms, 4),
                      # the other roof of the same kernel (its algorithmic bytes against the HBM peak)
                      "hbm_achieved_gbps": round(w["bytes_stage1"] / (g1_ms * 1e-3) / 1e9, 1),
                      "hbm_frac": round(w["bytes_stage1"] / (g1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)},
-        "decode": {"tokens": a.decode_tokens, "ms_per_step": round(dec["ms"], 4), "experts_hit": dw["e_hit"],
+        "decode": {"tokens": a.decode_tokens, "method": dec["method"], "block_m": dec["block_m"],
+                   "ms_per_step": round(dec["median_ms"], 4), "ms_iqr": [round(dec["q1_ms"], 4), round(dec["q3_ms"], 4)],
+                   "ms_wall_mean": round(dec["wall_ms"], 4), "experts_hit": dw["e_hit"],
                    "hbm_gbps": round(dec_gbps, 1), "frac_of_hbm_peak": round(dec_gbps / PEAK_HBM_GBPS, 4),
-                   "tflops": round(dw["flops"] / (dec["ms"] * 1e-3) / 1e12, 2),
-                   "stage_ms": {k: round(v, 4) for k, v in dec["stage_ms"].items()},
+                   "tflops": round(dw["flops"] / (dec["median_ms"] * 1e-3) / 1e12, 2),
+                   "stage_ms_untimed_pass": {k: round(v, 4) for k, v in dec_stage.items()},
                    "graph_replay_ms_per_step": round(dec_graph_ms, 4),
                    "roofline": {"kernel": "moe_gemm_w4a16_kernel<1,1> (gate_up, bf16 activations)", "bound": "hbm",
                                 "achieved": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                                 "unit": "GB/s",
                                 "frac": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                                "traffic": MEASURED_TRAFFIC.get((a.shape, a.decode_tokens)),
-                                "avg_launch_ms": round(dg1_ms, 4)}},
+                                "traffic": dtraffic, "avg_launch_ms": round(dg1_ms, 4)}},
+        "decode_a4w4": {"tokens": a.decode_tokens, "ms_per_step": round(dec4["median_ms"], 4),
+                        "hbm_gbps": round(dw["bytes"] / (dec4["median_ms"] * 1e-3) / 1e9, 1),
+                        "frac_of_hbm_peak": round(dw["bytes"] / (dec4["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)},
+        "configs": configs,
     }
-    out["decode_a4w4"] = {"tokens": a.decode_tokens, "ms_per_step": round(dec4["ms"], 4),
-                          "hbm_gbps": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9, 1),
-                          "frac_of_hbm_peak": round(dw["bytes"] / (dec4["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                          "stage_ms": {k: round(v, 4) for k, v in dec4["stage_ms"].items()}}
-    out["sweep"] = sweep
-    if a.cpu_seconds > 0:
-        out["cpu_baseline"] = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds)
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 

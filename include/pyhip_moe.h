@@ -165,6 +165,16 @@ int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t*
 int pyhip_moe_topk_reduce(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden, int out_is_f32,
                           const uint32_t* num_valid_ids, pyhip_stream_t stream);
 
+/* The same reduction with the routing in view: a slot is left out (neither read nor added) when the sort dropped
+ * its pair, i.e. when topk_ids[t, slot] is outside [0, experts), names an expert that expert_mask (device int32
+ * [experts], may be NULL) masks, or t >= *num_local_tokens (device int32 scalar, may be NULL); rows of tokens past
+ * the local count are written as zeros.  The down GEMMs write only the pairs that were sorted, so with this
+ * reduction out3 needs no clearing (the reference clears its output buffer inside the sorter instead,
+ * src/contrib/fused_moe.py:301-306) and under expert parallelism only the owned slots are read. */
+int pyhip_moe_topk_reduce_routed(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden, int out_is_f32,
+                                 const int32_t* topk_ids, int experts, const int32_t* expert_mask,
+                                 const int32_t* num_local_tokens, pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Zero fill of device memory with a kernel (safe inside a captured graph, where memset nodes are not).  The
  * reference zeroes its buffers with torch (src/contrib/fused_moe.py:306, moe_sorting's moe_buf). */

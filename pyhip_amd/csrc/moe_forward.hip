@@ -24,8 +24,8 @@ int pyhip_moe_gemm1_w4a16(const void*, const uint8_t*, const uint8_t*, const voi
                           const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, int, float, hipStream_t);
 int pyhip_moe_gemm2_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const float*,
                           const uint32_t*, const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, hipStream_t);
-int pyhip_moe_topk_reduce(const void*, void*, int64_t, int, int, int, const uint32_t*, hipStream_t);
-int pyhip_moe_zero_fill(void* p, int64_t bytes, hipStream_t stream);
+int pyhip_moe_topk_reduce_routed(const void*, void*, int64_t, int, int, int, const int32_t*, int, const int32_t*,
+                                 const int32_t*, hipStream_t);
 }
 
 namespace {
@@ -137,13 +137,6 @@ extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_str
                                      hidden_bf16, hidden_row_stride, tokens, hidden, ws + l.a1_q, ws + l.a1_s, stream);
     if(rc)
         return rc;
-    // slots routed to experts this rank does not hold, and tokens past the local count, contribute nothing
-    if(expert_mask || num_local_tokens)
-    {
-        rc = pyhip_moe_zero_fill(out3, (int64_t)tokens * topk * hidden * 2, stream);
-        if(rc)
-            return rc;
-    }
     if(w4a16)
     {
         rc = pyhip_moe_gemm1_w4a16(hidden_bf16, w1, w1_scale, bias1_bf16, s_ids, s_e, n_valid, ws + l.a2, tokens, topk,
@@ -165,5 +158,9 @@ extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_str
     }
     if(rc)
         return rc;
-    return pyhip_moe_topk_reduce(out3, out, tokens, topk, hidden, out_is_f32, nullptr, stream);
+    // Slots the sort dropped (ids outside [0, experts), experts this rank does not hold, tokens past the local count)
+    // were never written by the down GEMM: the reduction reads the routing and leaves them out, so out3 needs no
+    // clearing and the traffic under expert parallelism is that of the owned slots.
+    return pyhip_moe_topk_reduce_routed(out3, out, tokens, topk, hidden, out_is_f32, topk_ids, experts, expert_mask,
+                                        num_local_tokens, stream);
 }

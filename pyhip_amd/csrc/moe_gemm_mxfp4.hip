@@ -112,7 +112,10 @@ __device__ __forceinline__ void vm_load_b32(int& dst, int voff, v4i rsrc, int so
 }
 // global -> LDS without passing through registers: lane i's bytes land at lds_base + LDS_IMM + i * size.
 // (The hardware adds the instruction's immediate offset to the LDS address as well as to the global one, so
-// M0 is set to the target minus IMM.)
+// M0 is set to the target minus IMM.)  M0 cannot be named as a clobber: it is a reserved register for the compiler,
+// which neither tracks nor preserves it around inline assembly (it says so when asked to).  These helpers are sound
+// as long as the compiler's own code never uses M0 in these kernels (on gfx9 LDS instructions do not need it);
+// tests/test_build_checks.py checks on the generated code that nothing outside the inline assembly names M0.
 template <int IMM, int LDS_IMM>
 __device__ __forceinline__ void vm_dma_b128(int voff, v4i rsrc, int soff, u32 lds_base)
 {
@@ -737,6 +740,23 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
 #endif
 }
 
+// compute units of the current device (asked once per device, then remembered)
+static int device_cu_count()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 256;
+    int cus = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if(cus == 0)
+    {
+        if(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        __atomic_store_n(&cached[dev], cus, __ATOMIC_RELAXED);
+    }
+    return cus;
+}
+
 template <int STAGE>
 static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
 {
@@ -747,9 +767,7 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
     {
         // persistent: two workgroups per CU (one for 256-row tiles).  Small tiles would fit three or four; measured,
         // that changes nothing: they are bound by the weight stream
-        int dev = 0, cus = 256;
-        if(hipGetDevice(&dev) == hipSuccess)
-            (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        const int cus = device_cu_count();
         unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }

@@ -29,6 +29,43 @@ def _as_u8(t):
     return t if t.dtype == torch.uint8 else t.view(torch.uint8)
 
 
+def _require(cond, msg, exc=ValueError):
+    """argument checks raise (an ``assert`` would vanish under ``python -O``)"""
+    if not cond:
+        raise exc("fused_moe: " + msg)
+
+
+def _is_shuffled(w):
+    """the reference's convention (src/contrib/fused_moe.py:198-206): an ``nn.Parameter`` counts as pre-shuffled
+    (wrapping drops the attribute), otherwise the tensor attribute ``is_shuffled`` says so, default False"""
+    if isinstance(w, torch.nn.parameter.Parameter):
+        return True
+    return bool(getattr(w, "is_shuffled", False))
+
+
+_shuffle_cache = {}
+
+
+def _shuffled_u8(w):
+    """uint8 view of an MXFP4 weight tensor in the pre-shuffled layout the kernels read.  Plain-layout weights
+    ([E, N, K/2] row-major, ``is_shuffled`` unset) are shuffled once and remembered per storage (the reference's
+    kernels take both layouts, src/contrib/fused_moe.py:410,480; here the plain layout costs one re-tiling pass on
+    first use and a second copy of the weights)."""
+    wu = _as_u8(w)
+    if _is_shuffled(w):
+        return wu
+    from .mxfp4 import shuffle_weight
+    key = (wu.data_ptr(), tuple(wu.shape), str(wu.device))
+    hit = _shuffle_cache.get(key)
+    if hit is not None and hit[0] == wu._version:
+        return hit[1]
+    if len(_shuffle_cache) >= 16:
+        _shuffle_cache.clear()
+    out = shuffle_weight(wu.contiguous())
+    _shuffle_cache[key] = (wu._version, out)
+    return out
+
+
 def pick_block_m(tokens, topk, experts, hidden=0):
     """M-tile (= sort block size): the smallest tile that holds TWICE the expected rows per expert.  Every extra
     row block of an expert streams the expert's weights once more, and routing is uneven enough that a tile of just
@@ -41,13 +78,7 @@ def pick_block_m(tokens, topk, experts, hidden=0):
     tile one, read with non-temporal loads.  Its long epilogue only pays with a long K loop: DS-V3 (hidden 7168)
     T = 4096 / 5120 / 6144: 1.55 / 1.65 / 1.72 ms against 1.69 / 2.09 / 1.92 ms; the gpt-oss, Qwen3 and Mixtral shapes
     (hidden 3072 / 4096) lose 4-13 % with it at the same rows per expert."""
-    est = tokens * topk / max(experts, 1)
-    for bm in (16, 32, 64):
-        if 2 * est <= bm:
-            return bm
-    if hidden >= 6144 and 120 <= est <= 192:
-        return 256
-    return 128
+    return int(_lib.load().pyhip_moe_pick_block_m(tokens, topk, experts, hidden))
 
 
 def pick_w4a16(tokens, topk, experts, hidden):
@@ -58,16 +89,15 @@ def pick_w4a16(tokens, topk, experts, hidden):
     MXFP4-activation path, one workgroup per (row block, 256 output channels), cannot fill the GPU while the
     bf16-activation kernel splits K over four times as many workgroups (Mixtral shape up to 8 rows per expert,
     T = 1: 0.068 against 0.109 ms)."""
-    pairs = tokens * topk
-    sparse = 4 * pairs <= 3 * experts
-    few_tiles = min(pairs, experts) * (hidden // 256) < 512 and pairs <= 8 * experts
-    return sparse or few_tiles
+    return bool(_lib.load().pyhip_moe_pick_w4a16(tokens, topk, experts, hidden))
 
 
 def act_quant_mxfp4(x, rows_limit=None):
     """bf16 [rows, K] -> (uint8 [rows, K/2], uint8 [rows, ceil(K/512)*16]) in the GEMM's A-operand layout."""
     lib = _lib.load()
-    assert x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
+    _require(x.dtype == torch.bfloat16 and x.dim() == 2, "act_quant_mxfp4 takes a bf16 matrix", TypeError)
+    if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+        x = x.contiguous()
     rows, K = x.shape
     sk = lib.pyhip_moe_act_scale_stride(K)
     q = torch.empty(rows, K // 2, dtype=torch.uint8, device=x.device)
@@ -112,33 +142,42 @@ def fused_moe(
     ``activation=ActivationType.Swiglu`` selects gpt-oss's clamped SwiGLU with ``swiglu_limit`` (default 7.0, as
     tests/contrib/moe/test_moe.py:76-81)."""
     lib = _lib.load()
-    assert activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts"
+    _require(activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts only")
     act = 1 if activation == ActivationType.Swiglu else 0
     limit = float(swiglu_limit) if swiglu_limit else 7.0
-    assert quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path"
-    assert not doweight_stage1
-    assert a1_scale is None and a2_scale is None, "activations are quantised dynamically"
-    assert splitk in (0, 1, 4), "splitk: 0 = automatic, 1 = off, 4 = split K over the four waves (w4a16 path only)"
-    assert w1_scale is not None and w2_scale is not None
-    assert hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2
+    _require(quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path")
+    _require(not doweight_stage1, "doweight_stage1 is not supported (the reference rejects it as well)")
+    _require(a1_scale is None and a2_scale is None, "activations are quantised dynamically: a1_scale / a2_scale must be None")
+    _require(splitk in (0, 1, 4), "splitk: 0 = automatic, 1 = off, 4 = split K over the four waves (w4a16 path only)")
+    _require(w1_scale is not None and w2_scale is not None, "w1_scale and w2_scale (e8m0, shuffled) are required")
+    _require(hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2,
+             "hidden_states must be a bf16 matrix on the GPU", TypeError)
     out_dtype = hidden_states.dtype if dtype is None else dtype
-    assert out_dtype in (torch.bfloat16, torch.float32)
+    _require(out_dtype in (torch.bfloat16, torch.float32), "dtype must be bfloat16 or float32", TypeError)
+    _require(method in ("auto", "a4w4", "w4a16", "jit", "gluon"), "method=%r" % (method,))
 
-    w1u, w2u, w1s, w2s = _as_u8(w1), _as_u8(w2), _as_u8(w1_scale), _as_u8(w2_scale)
+    # weights in the plain layout (no ``is_shuffled`` mark) are re-tiled once; the scales always come e8m0-shuffled,
+    # as the reference passes them (tests/contrib/moe/test_moe.py:167-189)
+    w1u, w2u, w1s, w2s = _shuffled_u8(w1), _shuffled_u8(w2), _as_u8(w1_scale), _as_u8(w2_scale)
+    _require(w1u.dim() == 3 and w2u.dim() == 3, "w1 [E, 2*inter, hidden/2] and w2 [E, hidden, inter/2] expected")
     # hidden_pad / intermediate_pad: the weights arrive zero-padded to the kernels' tile multiples and the last
     # hidden_pad (intermediate_pad) channels are padding.  The activations may come at the padded width (the
     # reference's convention) or at the true width, in which case they are widened here and the result is
     # returned at the true width.
-    assert 0 <= hidden_pad < w1u.shape[2] * 2 and 0 <= intermediate_pad < w1u.shape[1] // 2
+    _require(0 <= hidden_pad < w1u.shape[2] * 2 and 0 <= intermediate_pad < w1u.shape[1] // 2, "bad hidden_pad / intermediate_pad")
     narrow = hidden_pad > 0 and hidden_states.shape[1] == w1u.shape[2] * 2 - hidden_pad
     if narrow:
         hidden_states = torch.nn.functional.pad(hidden_states, (0, hidden_pad))
     T, H = hidden_states.shape
+    _require(topk_ids.dim() == 2 and topk_ids.shape[0] == T and tuple(topk_weight.shape) == tuple(topk_ids.shape),
+             "topk_ids / topk_weight must be [tokens, topk]")
     k = topk_ids.shape[1]
     E, N1, Hb = w1u.shape
     I = N1 // 2
-    assert Hb * 2 == H and tuple(w2u.shape) == (E, H, I // 2), (w1u.shape, w2u.shape, H)
-    assert w1u.is_contiguous() and w2u.is_contiguous() and w1s.is_contiguous() and w2s.is_contiguous()
+    _require(Hb * 2 == H and tuple(w2u.shape) == (E, H, I // 2),
+             "shapes do not fit: hidden %d, w1 %s, w2 %s" % (H, tuple(w1u.shape), tuple(w2u.shape)))
+    _require(w1u.is_contiguous() and w2u.is_contiguous() and w1s.is_contiguous() and w2s.is_contiguous(),
+             "weights and scales must be contiguous")
     global_E = E if expert_mask is None else expert_mask.numel()
     dev = hidden_states.device
     if T == 0:
@@ -155,7 +194,6 @@ def fused_moe(
 
     topk_ids = topk_ids.to(torch.int32).contiguous()
     topk_weight = topk_weight.to(torch.float32).contiguous()
-    assert method in ("auto", "a4w4", "w4a16", "jit", "gluon")
     # "auto" (and the reference's "jit" / "gluon", which name its own back ends): see pick_w4a16
     w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, k, global_E, H))
     bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E, H)
@@ -163,21 +201,24 @@ def fused_moe(
         bm = min(bm, 64)
     if bias1 is not None:
         bias1 = bias1.to(torch.bfloat16).contiguous()
-        assert tuple(bias1.shape) == (E, 2 * I)
+        _require(tuple(bias1.shape) == (E, 2 * I), "bias1 must be [E, 2*inter]")
     if bias2 is not None:
         bias2 = bias2.to(torch.bfloat16).contiguous()
-        assert tuple(bias2.shape) == (E, H)
+        _require(tuple(bias2.shape) == (E, H), "bias2 must be [E, hidden]")
+
+    if expert_mask is not None:
+        expert_mask = expert_mask.to(device=dev, dtype=torch.int32).contiguous()
+    if num_local_tokens is not None:
+        _require(num_local_tokens.is_cuda and num_local_tokens.dtype == torch.int32,
+                 "num_local_tokens must be an int32 scalar tensor on the GPU", TypeError)
 
     if not return_parts and stage_events is None:
         # the whole layer in one library call, intermediates in one workspace: two allocations and one foreign call
         # per layer instead of a dozen of each (the host side is what bounds small layers when they are not replayed
         # from a graph)
-        if expert_mask is not None:
-            expert_mask = expert_mask.to(device=dev, dtype=torch.int32).contiguous()
-        if num_local_tokens is not None:
-            assert num_local_tokens.is_cuda and num_local_tokens.dtype == torch.int32
         x = hidden_states
-        if x.stride(1) != 1 or (w4a16 and x.stride(0) != H):
+        # the kernels read 16-byte pieces of a row: views with an odd row stride or base (a column slice) are copied
+        if x.stride(1) != 1 or (w4a16 and x.stride(0) != H) or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
             x = x.contiguous()
         ws_bytes = lib.pyhip_moe_forward_workspace_bytes(T, k, global_E, H, I, bm, 1 if w4a16 else 0)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
@@ -203,6 +244,13 @@ def fused_moe(
     n_blk = sorted_e.numel()
     stream = _lib.current_stream()
 
+    def _reduce(out3, out):
+        # slots the sort dropped (ids outside [0, E), masked experts, tokens past the local count) were never
+        # written by the down GEMM: the reduction reads the routing and leaves them out
+        return lib.pyhip_moe_topk_reduce_routed(_lib.dptr(out3), _lib.dptr(out), T, k, H,
+                                                1 if out_dtype == torch.float32 else 0, _lib.dptr(topk_ids), global_E,
+                                                _lib.dptr(expert_mask), _lib.dptr(num_local_tokens), stream)
+
     if w4a16:
         hs = hidden_states.contiguous()
         a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev)
@@ -212,16 +260,13 @@ def fused_moe(
         _lib.check(rc, "moe_gemm1_w4a16")
         ev = _mark("gemm1", ev)
         out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
-        if expert_mask is not None or num_local_tokens is not None:
-            out3.zero_()
         rc = lib.pyhip_moe_gemm2_w4a16(_lib.dptr(a2), _lib.dptr(w2u), _lib.dptr(w2s), _lib.dptr(bias2),
                                        _lib.dptr(sorted_ids), _lib.dptr(sorted_w), _lib.dptr(sorted_e),
                                        _lib.dptr(num_valid), _lib.dptr(out3), T, k, global_E, H, I, bm, n_blk, splitk, stream)
         _lib.check(rc, "moe_gemm2_w4a16")
         ev = _mark("gemm2", ev)
         out = torch.empty(T, H, dtype=out_dtype, device=dev)
-        rc = lib.pyhip_moe_topk_reduce(_lib.dptr(out3), _lib.dptr(out), T, k, H,
-                                       1 if out_dtype == torch.float32 else 0, None, stream)
+        rc = _reduce(out3, out)
         _lib.check(rc, "moe_topk_reduce")
         _mark("reduce", ev)
         if narrow:
@@ -243,8 +288,6 @@ def fused_moe(
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
     out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
-    if expert_mask is not None or num_local_tokens is not None:
-        out3.zero_()          # slots routed to experts this rank does not hold contribute nothing
     rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
                                    _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
                                    _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
@@ -252,8 +295,7 @@ def fused_moe(
     _lib.check(rc, "moe_gemm2_mxfp4")
     ev = _mark("gemm2", ev)
     out = torch.empty(T, H, dtype=out_dtype, device=dev)
-    rc = lib.pyhip_moe_topk_reduce(_lib.dptr(out3), _lib.dptr(out), T, k, H,
-                                   1 if out_dtype == torch.float32 else 0, None, stream)
+    rc = _reduce(out3, out)
     _lib.check(rc, "moe_topk_reduce")
     _mark("reduce", ev)
     if narrow:

@@ -60,7 +60,14 @@ def device_weights(L, dev="cuda"):
     w2 = torch.from_numpy(layout.shuffle_weight(L.w2q)).to(dev)
     w1s = torch.from_numpy(layout.e8m0_shuffle(L.w1s.reshape(L.E * 2 * L.I, L.H // 32))).to(dev)
     w2s = torch.from_numpy(layout.e8m0_shuffle(L.w2s.reshape(L.E * L.H, L.I // 32))).to(dev)
+    w1.is_shuffled = w2.is_shuffled = True        # the mark the operator looks for (src/contrib/fused_moe.py:198-206)
     return w1, w1s, w2, w2s
+
+
+def plain_device_weights(L, dev="cuda"):
+    """the same weights in the plain [E, N, K/2] layout (no ``is_shuffled`` mark); scales shuffled as always"""
+    w1, w1s, w2, w2s = device_weights(L, dev)
+    return torch.from_numpy(L.w1q).to(dev), w1s, torch.from_numpy(L.w2q).to(dev), w2s
 
 
 def padded_device_weights(L, dev="cuda"):
@@ -74,6 +81,7 @@ def padded_device_weights(L, dev="cuda"):
     w2 = torch.from_numpy(layout.shuffle_weight(w2q.numpy())).to(dev)
     s1 = torch.from_numpy(layout.e8m0_shuffle(w1s.numpy().reshape(E * 2 * Ip, Hp // 32))).to(dev)
     s2 = torch.from_numpy(layout.e8m0_shuffle(w2s.numpy().reshape(E * Hp, Ip // 32))).to(dev)
+    w1.is_shuffled = w2.is_shuffled = True
     return w1, s1, w2, s2, None if b1 is None else b1.to(dev), None if b2 is None else b2.to(dev), hp, ip
 
 

@@ -52,6 +52,27 @@ def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(gemm_asm):
         assert m and int(m.group(1)) == 0, (name, "spills")
 
 
+def test_compiler_never_uses_m0(gemm_asm):
+    """The LDS-DMA helpers set M0 by hand inside inline assembly.  M0 is reserved for the compiler (a clobber on it
+    is not honoured), so the helpers are only sound while no instruction of the compiler's own reads or writes M0
+    in these kernels."""
+    _, kernels = gemm_asm
+    for name, body in kernels:
+        inside, hand = False, 0
+        for line in body.split("\n"):
+            if "ASMSTART" in line:
+                inside = True
+            elif "ASMEND" in line:
+                inside = False
+            else:
+                code = line.split(";")[0]
+                if inside:
+                    hand += bool(re.search(r"\bm0\b", code))
+                else:
+                    assert not re.search(r"\bm0\b", code), (name, line)
+        assert hand, name
+
+
 def _instructions(body):
     for line in body.split("\n"):
         code = line.split(";")[0].strip()

@@ -1,9 +1,13 @@
-"""Full-size checks at the DeepSeek-V3 routed-expert shape (E=256, top-8, H=7168, I=2048), where the CPU oracle
-can only afford a sample: oracle parity on sampled experts plus size-independent properties of the layer.
+"""Every benchmark shape at its real size: Mixtral-8x7B (E=8, top-2, H=4096, I=14336), gpt-oss-120b (E=128, top-4,
+H=I=2880 padded to 3072, biases), Qwen3-235B-A22B (E=128, top-8, H=4096, I=1536, Zipf-skewed router) and
+DeepSeek-V3 (E=256, top-8, H=7168, I=2048, grouped sigmoid router), at the token counts the benchmark quotes.
+The CPU oracle can only afford a sample there: oracle parity on sampled experts plus size-independent properties
+of the layer.  (The reference's own shape sweep: tests/contrib/moe/test_moe.py:949-1035.)
 
-Floating-point tolerance: max|err| <= 1e-2 * rms(ref) (+ one bf16 ulp of the value for bf16 stage outputs),
-cosine >= 0.999.  The properties (token permutation, power-of-two scaling of the routing weights, top-k
-reduction as a checksum of the per-slot outputs) are bit-exact.
+Floating-point tolerance: max|err| <= 1e-2 * rms(ref) (+ one bf16 ulp of the value: both sides are bf16 roundings
+of nearly equal fp32 values), cosine >= 0.999, and the reference's own metric calc_diff <= 0.01
+(tests/contrib/moe/test_mxfp4.py:286-299).  The properties (token permutation, power-of-two scaling of the
+routing weights, top-k reduction as a checksum of the per-slot outputs, slot order) are bit-exact.
 """
 import numpy as np
 import pytest
@@ -13,68 +17,134 @@ from oracle import metrics, moe, mxfp4 as om
 
 pytestmark = pytest.mark.gpu
 
-SHAPE = "dsv3"
+# (shape, tokens, method).  "auto" is what the operator picks; where that is the bf16-activation family the
+# MXFP4-activation family is forced as well (and the other way round at the decode sizes of DeepSeek-V3).
+CASES = {
+    "mixtral": [(1, "auto"), (1, "a4w4"), (32, "auto"), (32, "a4w4"), (512, "auto"), (4096, "auto")],
+    "gptoss": [(16, "auto"), (16, "a4w4"), (256, "auto"), (4096, "auto")],
+    "qwen3": [(64, "auto"), (64, "w4a16"), (2048, "auto"), (8192, "auto")],
+    "dsv3": [(16, "auto"), (16, "a4w4"), (128, "auto"), (1024, "auto"), (8192, "auto"), (32768, "a4w4")],
+}
+SAMPLED_EXPERTS = {"mixtral": 1, "gptoss": 2, "qwen3": 2, "dsv3": 2}
 
 
 @pytest.fixture(scope="module")
-def layer():
+def layer(request):
+    """the weights of one benchmark shape (indirect parameter), generated once for all of that shape's cases"""
     from pyhip_amd import workloads
-    print("generating DS-V3-shaped weights on the device", flush=True)
-    W = workloads.make_weights(SHAPE)
+    shape = request.param
+    print(f"generating {shape}-shaped weights on the device", flush=True)
+    W = workloads.make_weights(shape)
+    W["shape"] = shape
     torch.cuda.synchronize()
-    return W
+    yield W
+    W.clear()
+    torch.cuda.empty_cache()
 
 
 def _run(W, hidden, tw, ti, **kw):
     from pyhip_amd import fused_moe
-    return fused_moe(hidden, W["w1"], W["w2"], tw, ti, w1_scale=W["w1_scale"], w2_scale=W["w2_scale"], **kw)
+    return fused_moe(hidden, W["w1"], W["w2"], tw, ti, w1_scale=W["w1_scale"], w2_scale=W["w2_scale"],
+                     bias1=W.get("bias1"), bias2=W.get("bias2"), hidden_pad=W["hidden_pad"],
+                     intermediate_pad=W["intermediate_pad"], **kw)
 
 
-@pytest.mark.parametrize("T,method", [(16, "w4a16"), (16, "a4w4"), (1024, "a4w4"), (8192, "a4w4"), (32768, "a4w4")])
+def _expert_f32(W, e, Hp, Ip):
+    """dequantised (padded) weights of one expert from the device tensors the operator reads"""
+    from pyhip_amd import mxfp4 as pm
+    w1 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w1"][e]).cpu().numpy(),
+                             W["w1_scale_plain"][e * 2 * Ip:(e + 1) * 2 * Ip].cpu().numpy())
+    w2 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w2"][e]).cpu().numpy(),
+                             W["w2_scale_plain"][e * Hp:(e + 1) * Hp].cpu().numpy())
+    return w1, w2
+
+
+def _cases():
+    return [pytest.param(s, T, m, id=f"{s}-T{T}-{m}") for s, lst in CASES.items() for T, m in lst]
+
+
+@pytest.mark.parametrize("layer,T,method", _cases(), indirect=["layer"])
 def test_sampled_experts_and_properties(layer, T, method):
-    from pyhip_amd import mxfp4 as pm, workloads
+    from pyhip_amd import workloads
+    from pyhip_amd.fused_moe import pick_w4a16
     W = layer
-    cfg = workloads.SHAPES[SHAPE]
+    shape = W["shape"]
+    cfg = workloads.SHAPES[shape]
     E, k, H, I = cfg["E"], cfg["k"], cfg["H"], cfg["I"]
-    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
-    print(f"full-size case {SHAPE} T={T} method={method}", flush=True)
-    a4 = method == "a4w4"
+    Hp, Ip = H + W["hidden_pad"], I + W["intermediate_pad"]
+    hidden, tw, ti = workloads.make_inputs(shape, T)
+    a4 = method == "a4w4" or (method == "auto" and not pick_w4a16(T, k, E, Hp))
+    print(f"full-size case {shape} T={T} method={method} ({'a4w4' if a4 else 'w4a16'})", flush=True)
     out, parts = _run(W, hidden, tw, ti, return_parts=True, method=method)
     out32 = _run(W, hidden, tw, ti, dtype=torch.float32, method=method)
     torch.cuda.synchronize()
-    out3 = parts["out3"]
-    assert torch.isfinite(out.float()).all()
+    assert out.shape == (T, H) and torch.isfinite(out.float()).all()
+    out3 = parts["out3"]                                              # [T, k, Hp]
 
     # (1) the top-k reduction is the fp32 sum of the per-slot outputs in slot order, rounded once
-    acc = torch.zeros(T, H, dtype=torch.float32, device="cuda")
+    acc = torch.zeros(T, Hp, dtype=torch.float32, device="cuda")
     for s in range(k):
         acc += out3[:, s].float()
-    assert torch.equal(out32, acc)
-    assert torch.equal(out, acc.to(torch.bfloat16))
+    assert torch.equal(out32, acc[:, :H])
+    assert torch.equal(out, acc[:, :H].to(torch.bfloat16))
+    assert (out3[:, :, H:] == 0).all()                                # padded channels stay zero
 
     # (2) oracle parity on sampled experts: per-(token, slot) outputs of the pairs routed to them
     ids = ti.cpu().numpy()
-    hit = np.unique(ids)
+    hit, counts = np.unique(ids, return_counts=True)
     rng = np.random.default_rng(T)
-    sample = rng.choice(hit, size=min(2, len(hit)), replace=False)
-    x = hidden.float().cpu().numpy()
+    sample = set(int(e) for e in rng.choice(hit, size=min(SAMPLED_EXPERTS[shape], len(hit)), replace=False))
+    if cfg["router"] == "zipf":
+        sample.add(int(hit[np.argmax(counts)]))                       # and the most loaded expert of the skewed router
+    x = np.zeros((T, Hp), np.float32)
+    x[:, :H] = hidden.float().cpu().numpy()
     xq = moe.act_quant_dequant(x) if a4 else x
     twn = tw.cpu().numpy()
-    for e in sample:
-        e = int(e)
-        w1 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w1"][e]).cpu().numpy(),
-                                 W["w1_scale_plain"][e * 2 * I:(e + 1) * 2 * I].cpu().numpy())
-        w2 = om.dequantize_mxfp4(pm.deshuffle_weight(W["w2"][e]).cpu().numpy(),
-                                 W["w2_scale_plain"][e * H:(e + 1) * H].cpu().numpy())
+    b1 = None if "bias1" not in W else W["bias1"].float().cpu().numpy()
+    b2 = None if "bias2" not in W else W["bias2"].float().cpu().numpy()
+    # sorted position of every (token, slot) pair
+    so = parts["sorted_ids"].cpu().numpy().view(np.uint32)
+    nv = int(parts["num_valid_ids"][0])
+    tok_p, slot_p = (so[:nv] & 0xFFFFFF).astype(np.int64), (so[:nv] >> 24).astype(np.int64)
+    real = slot_p < k
+    pos_of = np.full((T, k), -1, np.int64)
+    pos_of[tok_p[real], slot_p[real]] = np.nonzero(real)[0]
+    assert (pos_of >= 0).all()                                        # every pair was sorted exactly once
+    for e in sorted(sample):
+        w1, w2 = _expert_f32(W, e, Hp, Ip)
         t_idx, s_idx = np.nonzero(ids == e)
-        a2 = moe.gateup_ref(xq[t_idx], w1)
-        ref = moe.down_ref(moe.act_quant_dequant(a2) if a4 else a2, w2, twn[t_idx, s_idx])
+        if len(t_idx) > 1536:                                         # bounded CPU time: a sample of the expert's pairs
+            pick = np.sort(rng.choice(len(t_idx), size=1536, replace=False))
+            t_idx, s_idx = t_idx[pick], s_idx[pick]
+        a2 = moe.gateup_ref(xq[t_idx], w1, None if b1 is None else b1[e])
+        ref = moe.down_ref(moe.act_quant_dequant(a2) if a4 else a2, w2, twn[t_idx, s_idx], None if b2 is None else b2[e])
         got = out3[torch.from_numpy(t_idx).cuda(), torch.from_numpy(s_idx).cuda()].float().cpu().numpy()
+        # the kernel's own stage-1 rows of these pairs (a2 is indexed by sorted position)
+        got_a2 = parts["a2"][torch.from_numpy(pos_of[t_idx, s_idx]).cuda()].float().cpu().numpy()
+        rms1 = np.sqrt(np.mean(a2.astype(np.float64) ** 2))
+        e1 = np.abs(got_a2 - a2) - np.abs(a2) * 2.0 ** -7
+        nflip = int((got_a2 != a2).sum())
+        assert e1.max() <= 1e-2 * rms1, "stage 1 beyond one bf16 ulp"
         rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
-        err = np.abs(got - ref) - np.abs(ref) * 2.0 ** -7          # one bf16 ulp of the value
+        raw = np.abs(got - ref)
+        err = raw - np.abs(ref) * 2.0 ** -7          # one bf16 ulp of the value
         cos = metrics.cosine(got, ref)
-        print(f"  expert {e}: {len(t_idx)} pairs, (max|err| - ulp)/rms = {err.max() / rms:.3e}, cosine = {cos:.7f}", flush=True)
-        assert err.max() <= 1e-2 * rms and cos >= 0.999
+        cd = metrics.calc_diff(got, ref)
+        # the oracle's stage 2 on the kernel's own stage-1 result: isolates stage 2 from roundings of a2 that went the other way
+        ref_g = moe.down_ref(moe.act_quant_dequant(got_a2) if a4 else got_a2, w2, twn[t_idx, s_idx], None if b2 is None else b2[e])
+        err_g = np.abs(got - ref_g) - np.abs(ref_g) * 2.0 ** -7
+        print(f"  expert {e}: {len(t_idx)} pairs, stage-1 values rounded the other way: {nflip} of {a2.size}; "
+              f"max|err|/rms = {raw.max() / rms:.3e} (beyond one bf16 ulp: {max(err.max(), 0) / rms:.3e}, given the "
+              f"kernel's stage-1 result: {max(err_g.max(), 0) / rms:.3e}), fraction beyond 1e-2*rms = "
+              f"{np.mean(raw > 1e-2 * rms):.2e}, cosine = {cos:.7f}, calc_diff = {cd:.2e}", flush=True)
+        assert cos >= 0.999 and cd <= 0.01
+        assert err_g.max() <= 1e-2 * rms
+        if a4 and nflip:
+            # a stage-1 value that sits on a bf16 rounding boundary AND on an e2m1 boundary moves one re-quantised
+            # activation by a whole e2m1 step (tests/test_gpu_moe.py::_end_to_end): isolated outliers, bounded
+            assert np.mean(err > 1e-2 * rms) <= 2e-3 and err.max() <= 0.1 * rms
+        else:
+            assert err.max() <= 1e-2 * rms
 
     # (3) permuting the tokens permutes the output rows, bit for bit
     perm = torch.randperm(T, generator=torch.Generator().manual_seed(T)).cuda()
@@ -91,33 +161,43 @@ def test_sampled_experts_and_properties(layer, T, method):
     assert torch.equal(parts_r["out3"][:, rev], out3)
 
 
+TILE_CASES = {
+    # the token count at which the experts' row counts straddle a tile height: second blocks that are almost empty
+    "dsv3": (8192, (64, 128, 256)), "qwen3": (8192, (64, 128, 256)), "mixtral": (4096, (128, 256)),
+    "gptoss": (4096, (32, 128, 256)),
+}
+
+
+@pytest.mark.parametrize("layer", list(TILE_CASES), indirect=True)
 def test_tile_heights_agree_bit_for_bit(layer):
-    """128-row and 256-row tiles compute every routed row with the same instructions in the same order, so the
-    layer output must not depend on block_size_M.  At T=8192 about half of the experts have a few rows more than
-    256: their second 256-row block is almost empty, its K-groups are short, and every hand-counted wait of the
-    pipeline really has to hold (a data race in the 256-row tile showed up exactly there)."""
+    """Every tile height computes every routed row with the same instructions in the same order, so the layer output
+    must not depend on block_size_M.  Where experts have a few rows more than a tile holds, their last block is
+    almost empty, its K-groups are short, and every hand-counted wait of the pipeline really has to hold (a data
+    race in the 256-row tile showed up exactly there)."""
     W = layer
-    T = 8192
     from pyhip_amd import workloads
-    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
-    print(f"full-size case {SHAPE} T={T} block_size_M 64 / 128 / 256", flush=True)
-    outs = {bm: _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm) for bm in (64, 128, 256)}
+    shape = W["shape"]
+    T, bms = TILE_CASES[shape]
+    hidden, tw, ti = workloads.make_inputs(shape, T)
+    print(f"full-size case {shape} T={T} block_size_M {bms}", flush=True)
+    outs = {bm: _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm) for bm in bms}
     torch.cuda.synchronize()
-    assert torch.isfinite(outs[128].float()).all()
-    assert torch.equal(outs[64], outs[128])
-    assert torch.equal(outs[256], outs[128])
+    assert torch.isfinite(outs[bms[0]].float()).all()
+    for bm in bms[1:]:
+        assert torch.equal(outs[bm], outs[bms[0]]), bm
 
 
+@pytest.mark.parametrize("layer", ["dsv3"], indirect=True)
 @pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 256))])
 def test_load_policies_agree_bit_for_bit(layer, T, bms):
     """The launch marks the weight loads non-temporal while the rows per expert stay under three quarters of a row
-    block (T=1024: 32 rows per expert, so the 64-, 128- and 256-row tiles take that instance and the 16- and 32-row
-    tiles the other; T=4096: 128 rows per expert, only the 256-row tile does).  A cache policy must not change a
-    bit of the result."""
+    block (DeepSeek-V3 shape, T=1024: 32 rows per expert, so the 64-, 128- and 256-row tiles take that instance and
+    the 16- and 32-row tiles the other; T=4096: 128 rows per expert, only the 256-row tile does).  A cache policy
+    must not change a bit of the result."""
     W = layer
     from pyhip_amd import workloads
-    hidden, tw, ti = workloads.make_inputs(SHAPE, T)
-    print(f"full-size case {SHAPE} T={T} block_size_M {bms}", flush=True)
+    hidden, tw, ti = workloads.make_inputs("dsv3", T)
+    print(f"full-size case dsv3 T={T} block_size_M {bms}", flush=True)
     outs = {bm: _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm) for bm in bms}
     torch.cuda.synchronize()
     assert torch.isfinite(outs[bms[0]].float()).all()

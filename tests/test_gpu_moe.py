@@ -48,7 +48,8 @@ def test_act_quant_bit_exact():
 
 def _stage_checks(L, parts, bm):
     """stage-by-stage comparison; every stage is fed the KERNEL's previous output.
-    -> (worst stage-1 error, worst stage-2 error, the oracle's layer output given the kernel's stage-1 result)"""
+    -> (worst stage-1 error, worst stage-2 error, the oracle's layer output given the kernel's stage-1 result,
+        numbers of stage-1 / stage-2 values whose bf16 rounding went the other way than the oracle's)"""
     so = parts["sorted_ids"].cpu().numpy().view(np.uint32)
     se = parts["sorted_expert_ids"].cpu().numpy().view(np.uint32)
     sw = parts["sorted_weights"].cpu().numpy()
@@ -89,10 +90,12 @@ def _stage_checks(L, parts, bm):
     ref_out = np.zeros((L.T, out3.shape[2]), np.float32)
     for s in range(L.k):
         ref_out += per_slot[:, s]
-    return worst1, worst2, ref_out
+    print(f"  stage outputs that differ from the oracle's by a rounding: stage 1 {nflip1} of {ntot1}, "
+          f"stage 2 {nflip2} of {ntot2}; worst beyond one bf16 ulp: {worst1:.2e} / {worst2:.2e} of the rms", flush=True)
+    return worst1, worst2, ref_out, (nflip1, nflip2)
 
 
-def _end_to_end(got32, ref, ref_given_a2):
+def _end_to_end(got32, ref, ref_given_a2, nflip1):
     """The layer output against the oracle.  Both sides round the stage-1 result to bf16 and re-quantise it to
     MXFP4; two correct fp32 evaluation orders can round a value that sits on a bf16 boundary differently, and
     when that value also sits on an e2m1 boundary the re-quantised activation moves by a whole e2m1 step,
@@ -100,15 +103,26 @@ def _end_to_end(got32, ref, ref_given_a2):
     cosine >= 0.999) is asserted against the oracle evaluated from the kernel's own stage-1 result (whose
     one-ulp agreement with the oracle's is asserted separately), and against the pure oracle the same bound
     must hold for all but 2e-3 of the elements (one moved activation touches every output channel of its
-    row) with no error above 0.1 * rms."""
+    row) with no error above 0.1 * rms.  When no stage output was rounded the other way (nflip1 == (0, 0)) there
+    is nothing to excuse, and the strict bound is asserted against the pure oracle as well.  The reference's own
+    metric, calc_diff <= 0.01 for the MXFP4-activation path (tests/contrib/moe/test_mxfp4.py:286-299), is asserted
+    in every case."""
     err_a2, cos_a2 = metrics.max_err_over_rms(got32, ref_given_a2), metrics.cosine(got32, ref_given_a2)
     err, cos = metrics.max_err_over_rms(got32, ref), metrics.cosine(got32, ref)
     rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
     frac = float((np.abs(got32 - ref) > TOL_MAX * rms).mean())
     print(f"  vs oracle: max|err|/rms={err:.3e} cosine={cos:.8f} beyond-bound fraction={frac:.2e}; "
           f"given the kernel's a2: max|err|/rms={err_a2:.3e} cosine={cos_a2:.8f}", flush=True)
+    cd = metrics.calc_diff(got32, ref)
+    print(f"  calc_diff={cd:.3e}; strict bound against the pure oracle "
+          f"{'asserted (no stage rounding differs)' if not any(nflip1) else 'relaxed (%d stage-1, %d stage-2 roundings differ): worst %.3e of the 0.1 allowed, fraction %.2e of the 2e-3 allowed' % (nflip1[0], nflip1[1], err, frac)}",
+          flush=True)
     assert err_a2 <= TOL_MAX and cos_a2 >= TOL_COS
-    assert cos >= TOL_COS and frac <= 2e-3 and err <= 0.1
+    assert cd <= 0.01
+    if not any(nflip1):
+        assert err <= TOL_MAX and cos >= TOL_COS
+    else:
+        assert cos >= TOL_COS and frac <= 2e-3 and err <= 0.1
     return err
 
 
@@ -157,7 +171,7 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
     assert (q2.cpu().numpy() == oq2).all() and (cases.untranspose_act_scales(s2.cpu().numpy(), L.I) == os2).all()
 
     # stage-wise, each stage fed the kernel's own previous output
-    w1e, w2e, ref_a2 = _stage_checks(L, parts, parts["block_m"])
+    w1e, w2e, ref_a2, nflip1 = _stage_checks(L, parts, parts["block_m"])
     assert w1e <= TOL_MAX, f"stage 1 (max|err| - ulp)/rms = {w1e}"
     assert w2e <= TOL_MAX, f"stage 2 (max|err| - ulp)/rms = {w2e}"
 
@@ -166,8 +180,7 @@ def test_fused_moe_matches_oracle(name, T, bm, bias):
                       bias1=None if L.bias1 is None else _f(L.bias1), bias2=None if L.bias2 is None else _f(L.bias2))
     rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
     got32 = _f(out32)
-    _end_to_end(got32, ref, ref_a2)
-    print(f"  calc_diff={metrics.calc_diff(got32, ref):.3e}", flush=True)
+    _end_to_end(got32, ref, ref_a2, nflip1)
     half_ulp = np.abs(ref_a2) * 2.0 ** -8
     assert (np.abs(_f(out16) - ref_a2) <= TOL_MAX * rms + half_ulp).all()
     # the bf16 output is the rounding of the fp32 output
@@ -198,9 +211,9 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     nv = int(parts["num_valid_ids"][0])                   # rows past the padded total are never written
     assert (_f(parts["a2"])[:nv, L.I:] == 0).all() and (_f(parts["out3"])[:, :, L.H:] == 0).all()
     view = dict(parts, a2=parts["a2"][:, :L.I], out3=parts["out3"][:, :, :L.H])
-    w1e, w2e, ref_a2 = _stage_checks(L, view, parts["block_m"])
+    w1e, w2e, ref_a2, nflip1 = _stage_checks(L, view, parts["block_m"])
     assert w1e <= TOL_MAX and w2e <= TOL_MAX
-    _end_to_end(_f(out_narrow), ref, ref_a2)
+    _end_to_end(_f(out_narrow), ref, ref_a2, nflip1)
 
 
 @pytest.mark.parametrize("name,T,bm,bias,splitk", [
@@ -242,8 +255,14 @@ def test_w4a16_matches_oracle(name, T, bm, bias, splitk):
     ulp = np.abs(slot_ref).sum(axis=1) * 2.0 ** -7
     excess = np.maximum(np.abs(_f(out32) - ref) - ulp, 0).max() / rms
     err, cos = metrics.max_err_over_rms(_f(out32), ref), metrics.cosine(_f(out32), ref)
-    print(f"  max|err|/rms={err:.3e} (beyond the rounding allowance: {excess:.3e}) cosine={cos:.8f}", flush=True)
-    assert excess <= TOL_MAX and cos >= TOL_COS
+    # The allowance is needed because a slot value near 3 * rms carries a bf16 ulp of 2^-7 * 3 * rms = 2.3e-2 * rms
+    # by itself: one rounding that goes the other way already exceeds 1e-2 * rms, with both sides correct.  It is
+    # only ever used by a vanishing fraction of the elements, which is asserted (and printed) here.
+    beyond = float((np.abs(_f(out32) - ref) > TOL_MAX * rms).mean())
+    cd = metrics.calc_diff(_f(out32), ref)
+    print(f"  max|err|/rms={err:.3e} (beyond the rounding allowance: {excess:.3e}; fraction of elements beyond the "
+          f"strict bound: {beyond:.2e}) cosine={cos:.8f} calc_diff={cd:.3e}", flush=True)
+    assert excess <= TOL_MAX and cos >= TOL_COS and beyond <= 1e-3 and cd <= 0.01
 
 
 @pytest.mark.parametrize("method,limit,T", [("a4w4", None, 300), ("a4w4", 1.0, 37), ("w4a16", None, 20), ("w4a16", 0.5, 20)])
@@ -388,14 +407,15 @@ def test_expert_mask_and_local_tokens(method, T):
     for parity in (0, 1):
         mask = torch.tensor([(e % 2) == parity for e in range(E)], dtype=torch.int32, device="cuda")
         keep = mask.bool()
-        out, p = fused_moe(hidden, w1[keep].contiguous(), w2[keep].contiguous(), tw, ti, expert_mask=mask,
+        w1k, w2k = w1[keep].contiguous(), w2[keep].contiguous()
+        w1k.is_shuffled = w2k.is_shuffled = True
+        out, p = fused_moe(hidden, w1k, w2k, tw, ti, expert_mask=mask,
                            w1_scale=s1[keep].contiguous().view(-1, w1s.shape[-1]),
                            w2_scale=s2[keep].contiguous().view(-1, w2s.shape[-1]),
                            dtype=torch.float32, return_parts=True, method=method, block_size_M=16)
         torch.cuda.synchronize()
         mine = keep[ti.long()]                                   # [T, k]
-        assert torch.equal(p["out3"][mine], pf["out3"][mine])
-        assert (p["out3"][~mine] == 0).all()
+        assert torch.equal(p["out3"][mine], pf["out3"][mine])      # (slots owned elsewhere are never written nor read)
         total += out
     assert torch.allclose(total, full, rtol=1e-5, atol=1e-6)
 
@@ -450,3 +470,78 @@ def test_one_call_path_equals_the_step_by_step_path(name, T, method, bias):
     b, _ = fused_moe(hidden, w1, w2, tw, ti, num_local_tokens=nl, return_parts=True, **kw)
     torch.cuda.synchronize()
     assert torch.equal(a, b) and (a[T // 2:] == 0).all()
+
+
+def _poison_allocator(nbytes):
+    """NaN patterns into memory the caching allocator will hand out next, so that anything read without having
+    been written shows"""
+    junk = torch.full((nbytes // 2,), float("nan"), dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    del junk
+
+
+@pytest.mark.parametrize("method,T,one_call", [("a4w4", 90, True), ("a4w4", 90, False), ("w4a16", 7, True), ("w4a16", 7, False)])
+def test_dropped_pairs_contribute_exactly_zero(method, T, one_call):
+    """Ids outside [0, E) (a -1 or E sentinel for experts held elsewhere, the router's 0x7FFFFFFF for a NaN row) are
+    dropped by the sort, with no expert mask given: their slots are never written by the down GEMM and must
+    contribute exactly nothing, whatever the intermediate buffers held before.  The result equals the run in which
+    those slots carry a valid id and weight 0 ... except that no product is formed at all: compare with the
+    oracle, and bit for bit with the same call on buffers that held other garbage."""
+    L = cases.make_layer("dsv3_s", T, seed=21)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    ids = L.topk_ids.copy()
+    rng = np.random.default_rng(5)
+    drop = rng.random(ids.shape) < 0.3
+    ids[drop] = rng.choice(np.array([-1, L.E, L.E + 7, 0x7FFFFFFF], dtype=np.int64), size=int(drop.sum())).astype(np.int32)
+    ids[0, :] = -1                                               # a token with no expert at all: a zero row
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(ids).cuda()
+    print(f"dropped-pairs case dsv3_s T={T} method={method} one_call={one_call}", flush=True)
+    kw = dict(w1_scale=w1s, w2_scale=w2s, dtype=torch.float32, method=method, block_size_M=16)
+    outs = []
+    for fill in (0, 1):
+        _poison_allocator(64 << 20) if fill else torch.zeros(32 << 20, dtype=torch.uint8, device="cuda")
+        o = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, **kw) if one_call else \
+            fused_moe(L.hidden.cuda(), w1, w2, tw, ti, return_parts=True, **kw)[0]
+        torch.cuda.synchronize()
+        outs.append(o.clone())
+    assert torch.isfinite(outs[1]).all() and torch.equal(outs[0], outs[1])
+    assert (outs[1][0] == 0).all()
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, ids, act="a4" if method == "a4w4" else "a16")
+    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+    err = np.abs(_f(outs[1]) - ref) / rms
+    print(f"  max|err|/rms={err.max():.3e} beyond-bound fraction={np.mean(err > TOL_MAX):.2e}", flush=True)
+    assert np.mean(err > TOL_MAX) <= 2e-3 and err.max() <= 0.1 and metrics.cosine(_f(outs[1]), ref) >= TOL_COS
+
+
+@pytest.mark.parametrize("method,T", [("a4w4", 50), ("w4a16", 5)])
+def test_plain_layout_weights(method, T):
+    """Weights without the ``is_shuffled`` mark are in the plain [E, N, K/2] layout (the reference's kernels take
+    both, src/contrib/fused_moe.py:198-206,410,480): the operator re-tiles them once and gives the same bits."""
+    L = cases.make_layer("tiny", T, seed=13)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    p1, _, p2, _ = cases.plain_device_weights(L)
+    assert not getattr(p1, "is_shuffled", False)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    print(f"plain-layout case tiny T={T} method={method}", flush=True)
+    a = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+    b = fused_moe(L.hidden.cuda(), p1, p2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+    c = fused_moe(L.hidden.cuda(), torch.nn.Parameter(w1.clone(), requires_grad=False),
+                  torch.nn.Parameter(w2.clone(), requires_grad=False), tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and torch.equal(a, c)
+
+
+def test_odd_views_of_hidden_states_are_copied():
+    """a column slice at an odd element offset (base not 16-byte aligned, row stride not a multiple of 8) is made
+    contiguous instead of being refused"""
+    L = cases.make_layer("tiny", 12, seed=14)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    wide = torch.zeros(12, L.H + 5, dtype=torch.bfloat16, device="cuda")
+    wide[:, 3:3 + L.H] = L.hidden.cuda()
+    view = wide[:, 3:3 + L.H]
+    for method in ("a4w4", "w4a16"):
+        a = fused_moe(view, w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+        b = fused_moe(view.contiguous(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
