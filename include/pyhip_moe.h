@@ -205,6 +205,23 @@ int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const 
                       int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
                       void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
 
+/* pyhip_moe_forward without the workspace argument: the intermediates live in a device array that belongs to the
+ * library (64 MiB, pyhip_moe_forward_static_capacity(); one copy per GPU, held until the process ends).  It has no
+ * counterpart in the reference.  It is for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates nothing (no hipMalloc, no
+ * hipFree, no allocating library routine); calls whose intermediates exceed the capacity are refused with error 1
+ * before anything is launched (decode-sized calls fit: DeepSeek-V3 shape, 128 tokens, bf16 activations: 35 MiB).
+ * Same arguments, kernels and results as pyhip_moe_forward.  All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams, two threads) race; nothing in the array needs clearing between calls. */
+int64_t pyhip_moe_forward_static_capacity(void);
+int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
+                             const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                             const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
+                             const float* topk_weights, const int32_t* expert_mask, const int32_t* num_local_tokens,
+                             void* out, int out_is_f32, int tokens, int topk, int experts, int hidden, int inter,
+                             int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
+                             pyhip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
