@@ -269,7 +269,13 @@ def main():
                 continue
             steps, warm = (a.steps, a.warmup) if t >= 1024 else (max(a.steps, 50), max(a.warmup, 10))
             r = time_point(torch, fused_moe, W, s, t, steps, warm, 0, "auto")
-            configs.append(point_record(s, t, r))
+            rec = point_record(s, t, r)
+            # where the time goes: launch groups of the step-by-step path, from events in a separate untimed pass
+            if rec["method"] == "a4w4" and rec["block_m"] >= 64:
+                # how evenly the persistent GEMMs' tiles spread over the 8 XCDs for this routing
+                rec["gate_up_tiles_per_xcd"] = workloads.xcd_tile_counts(s, r["topk_ids"], rec["block_m"], W["intermediate_pad"])
+            rec["stage_ms_untimed_pass"] = {k: round(v, 4) for k, v in stage_pass(torch, fused_moe, W, r, 0, "auto", 4).items()}
+            configs.append(rec)
             del r
         if shape == a.shape:
             # headline: exactly --steps timed calls after --warmup untimed ones

@@ -58,11 +58,12 @@ int pyhip_moe_topk_grouped_sigmoid(const float* gating, int tokens, int experts,
  * num_local_tokens (device int32 scalar, may be NULL) limits the tokens that are read.
  * moe_out (may be NULL) is zero-filled over moe_out_bytes, as the reference's sorter does for the
  * layer output.  workspace: pyhip_moe_sorting_workspace_bytes() bytes of device memory.
- * schedule (may be NULL; pyhip_moe_schedule_words(experts) u32 words) receives the tile schedule the
- * grouped GEMMs below walk as a persistent grid: experts are dealt to the 8 XCDs (e % 8) and every
- * XCD gets the prefix sums of its experts' row-block counts plus each expert's first row block.  It has
- * no counterpart in the reference, which launches one workgroup per (tile, worst-case block)
- * (src/contrib/moe_gemm_mxfp4.py:1000-1011). */
+ * schedule (may be NULL; pyhip_moe_schedule_words(experts) = 2 * experts + 1 u32 words) receives the table the
+ * grouped GEMMs below walk as a persistent grid: schedule[e], e = 0..experts, is the number of row blocks of
+ * the experts before e, schedule[experts + 1 + e] the local id of expert e.  A GEMM orders its tiles expert ->
+ * weight tile -> row block and gives each of the 8 XCDs an equal run of that list, so skewed expert loads still
+ * fill every XCD.  It has no counterpart in the reference, which launches one workgroup per (tile, worst-case
+ * block) (src/contrib/moe_gemm_mxfp4.py:1000-1011). */
 int64_t pyhip_moe_sorting_max_blocks(int64_t tokens, int topk, int experts, int block_size);
 int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, int experts);
 int64_t pyhip_moe_schedule_words(int experts);

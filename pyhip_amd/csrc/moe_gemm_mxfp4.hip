@@ -179,7 +179,9 @@ struct TileId
     bool valid;
 };
 
-#define SCHED_EX_MAX (2048 / 8 + 2)
+// most experts a persistent launch can serve: the schedule (E + 1 block prefixes, E local ids) sits in LDS next to the
+// activation stages, and two workgroups of the 128-row tile must still fit one CU (2 x 80 KB)
+#define SCHED_E_MAX 704
 
 // STAGE 1 = gate_up, 2 = down.  MT = row groups of 16 per tile.
 //
@@ -222,9 +224,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     __shared__ __attribute__((aligned(16))) uint8_t lds_s1[SLOTS * 256];
     __shared__ u32 lds_meta[3][2 * MPAD];     // per tile: sorted ids | routing weights; ring of 3 tiles
     __shared__ u32 lds_dummy[64];             // where the zeros of switched-off meta DMA operations land
-    __shared__ u32 lds_pre[SCHED_EX_MAX];     // this XCD's schedule: block-count prefix,
-    __shared__ u32 lds_first[SCHED_EX_MAX];   //   first row block and
-    __shared__ u32 lds_lid[SCHED_EX_MAX];     //   local id of its experts
+    __shared__ u32 lds_pre[SCHED_E_MAX + 1];  // the schedule: row blocks before every expert (and their total),
+    __shared__ u32 lds_lid[SCHED_E_MAX];      //   local id of every expert
 
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);   // wave-uniform: keeps descriptors and LDS bases scalar
@@ -234,25 +235,26 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     const int KS = g.K / 512;
     const int I  = g.N / 2;   // stage 1 only
 
-    // ---- tile iterator.  With a schedule the grid is persistent: workgroup w serves XCD x = w % 8 (the
-    // hardware deals consecutive workgroup ids round-robin to the XCDs) and walks that XCD's tile list
-    // with stride gridDim/8; the list is ordered expert -> weight tile -> row block, so the row blocks
-    // that share a weight tile run next to each other and every expert's data stays in one L2.
+    // ---- tile iterator.  With a schedule the grid is persistent.  All tiles, ordered expert -> weight tile -> row
+    // block (the row blocks that share a weight tile next to each other), form one list; it is cut into 8 equal
+    // runs, one per XCD, so every XCD (its own L2) gets the same number of tiles however unevenly the router loads
+    // the experts, and an expert's data still meets in one L2 (two where a cut falls inside an expert).  Workgroup w
+    // serves XCD w % 8 (the hardware deals consecutive workgroup ids round-robin to the XCDs) and walks that XCD's
+    // run with stride gridDim/8.
     // Without a schedule (or when K has a single K-group): one tile per workgroup, weight tile fastest.
     const bool persistent = g.sched != nullptr;
-    const int EX          = g.E / 8 + 2;
     const int xcd         = blockIdx.x & 7;
     const u32 qstride     = gridDim.x >> 3;
     u32 q                 = blockIdx.x >> 3;
-    int ei                = 0;                        // cursor into this XCD's expert list (q only grows)
+    u32 q_end             = 0;
+    int ei                = 0;                        // cursor into the expert list (q only grows)
     if(persistent)
     {
-        for(int i = tid; i < EX; i += GEMM_THREADS)
+        for(int i = tid; i <= g.E; i += GEMM_THREADS)
         {
-            const int e  = xcd + 8 * i;
-            lds_pre[i]   = g.sched[xcd * EX + i];
-            lds_first[i] = e < g.E ? g.sched[8 * EX + e] : 0u;
-            lds_lid[i]   = e < g.E ? g.sched[8 * EX + g.E + e] : 0u;
+            lds_pre[i] = g.sched[i];
+            if(i < g.E)
+                lds_lid[i] = g.sched[g.E + 1 + i];
         }
         __syncthreads();
     }
@@ -261,11 +263,32 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         return (v4i){__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y),
                      __builtin_amdgcn_readfirstlane(v.z), __builtin_amdgcn_readfirstlane(v.w)};
     };
+    if(persistent)
+    {
+        const u32 tiles = uni(lds_pre[g.E]) * (u32)g.n_tiles;
+        const u32 chunk = (tiles + 7u) >> 3;
+        q += (u32)xcd * chunk;
+        q_end = (u32)(xcd + 1) * chunk < tiles ? (u32)(xcd + 1) * chunk : tiles;
+        if(q < q_end)
+        {
+            // first expert whose tiles end beyond q
+            int lo = 0, hi = g.E - 1;
+            while(lo < hi)
+            {
+                const int mid = (lo + hi) >> 1;
+                if(uni(lds_pre[mid + 1]) * (u32)g.n_tiles > q)
+                    hi = mid;
+                else
+                    lo = mid + 1;
+            }
+            ei = lo;
+        }
+    }
     auto decode = [&](TileId& t) __attribute__((always_inline)) {
         t.valid = false;
         if(persistent)
         {
-            if(q >= uni(lds_pre[EX - 1]) * (u32)g.n_tiles)
+            if(q >= q_end)
                 return;
             while(q >= uni(lds_pre[ei + 1]) * (u32)g.n_tiles)
                 ei++;
@@ -273,7 +296,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             const u32 nb    = uni(lds_pre[ei + 1]) - p0;
             const u32 local = q - p0 * (u32)g.n_tiles;
             t.nt            = (int)(local / nb);
-            t.m_blk         = (int)(uni(lds_first[ei]) + (local - (u32)t.nt * nb));
+            t.m_blk         = (int)(p0 + (local - (u32)t.nt * nb));
             t.e             = (int)uni(lds_lid[ei]);
             q += qstride;
         }
@@ -761,8 +784,9 @@ template <int STAGE>
 static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
 {
     unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
-    if(g.K < 1024)
-        g.sched = nullptr;   // a single K-group per tile: no room to prefetch across tiles, one tile per workgroup
+    if(g.K < 1024 || g.E > SCHED_E_MAX)
+        g.sched = nullptr;   // a single K-group per tile (no room to prefetch across tiles) or more experts than the
+                             // schedule table in LDS holds: one tile per workgroup
     if(g.sched)
     {
         // persistent: two workgroups per CU (one for 256-row tiles).  Small tiles would fit three or four; measured,

@@ -252,46 +252,24 @@ __device__ __forceinline__ void fill_blocks(const SortArgs& a, const u32* tot, c
     }
 }
 
-// Tile schedule for the persistent grouped GEMMs.  Experts are dealt to the 8 XCDs (expert e -> XCD e % 8)
-// so that all row blocks and weight tiles of an expert meet in one L2.  Layout (u32 words), EX = E/8 + 2:
-//   sched[x*EX + i], i = 0..EX-1 : number of row blocks owned by the first i experts of XCD x
-//                                  (experts x, x+8, x+16, ...; entries past the last expert repeat the total)
-//   sched[8*EX + e]              : first row block of expert e
-//   sched[8*EX + E + e]          : local id of expert e (its index among the unmasked experts)
-// One workgroup; uses the first 8 waves.
-__device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* tot, const u32* off, const u32* lid)
+// Tile schedule for the persistent grouped GEMMs: the table from which every workgroup finds its tiles without
+// looking at sorted_expert_ids.  Layout (u32 words):
+//   sched[e], e = 0..E   : number of row blocks of the experts before e (sched[E] = all row blocks); the row blocks
+//                          of expert e are sched[e] .. sched[e+1]-1
+//   sched[E + 1 + e]     : local id of expert e (its index among the unmasked experts)
+// A GEMM orders its tiles expert -> weight tile -> row block and cuts that list into 8 equal runs, one per XCD
+// (moe_gemm_mxfp4.hip), so the XCDs get the same number of tiles however unevenly the router loads the experts.
+__device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* off, const u32* lid, u32 padded_total)
 {
     if(!a.sched)
         return;
-    const int EX   = a.E / 8 + 2;
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
-    if(wave < 8)
-    {
-        u32 run = 0;
-        for(int i0 = 0; i0 < EX; i0 += WAVE)
-        {
-            const int i = i0 + lane;
-            const int e = wave + 8 * i;
-            u32 nb      = 0;
-            if(i < EX && e < a.E && (!a.expert_mask || a.expert_mask[e] != 0))
-                nb = (tot[e] + a.Bm - 1) / a.Bm;
-            u32 sc = nb;
-            for(int d = 1; d < WAVE; d <<= 1)
-            {
-                u32 t = __shfl_up(sc, d);
-                if(lane >= d)
-                    sc += t;
-            }
-            if(i < EX)
-                a.sched[wave * EX + i] = run + sc - nb;
-            run += __shfl(sc, WAVE - 1);
-        }
-    }
     for(int e = threadIdx.x; e < a.E; e += blockDim.x)
     {
-        a.sched[8 * EX + e]       = off[e] / a.Bm;
-        a.sched[8 * EX + a.E + e] = lid[e];
+        a.sched[e]           = off[e] / a.Bm;
+        a.sched[a.E + 1 + e] = lid[e];
     }
+    if(threadIdx.x == 0)
+        a.sched[a.E] = padded_total / a.Bm;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -342,7 +320,7 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kerne
     __syncthreads();
     u32 padded_total = expert_offsets(a, tot, off, lid, scratch);
     fill_blocks(a, tot, off, lid, padded_total, T);
-    write_schedule(a, tot, off, lid);
+    write_schedule(a, off, lid, padded_total);
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         for(int w = 0; w < SMALL_WAVES; w++)
             whist[w * a.E + e] += off[e];
@@ -420,7 +398,7 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_scan_kernel
     for(int e = threadIdx.x; e < a.E; e += SMALL_THREADS)
         g_off[e] = off[e];
     fill_blocks(a, tot, off, lid, padded_total, T);
-    write_schedule(a, tot, off, lid);
+    write_schedule(a, off, lid, padded_total);
 }
 
 // launch 3 of 3: scatter.  LDS: whist[SORT_WAVES][E]
@@ -520,7 +498,7 @@ extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, i
     return ((int64_t)sort_groups(pairs) + 1) * experts * 4 + 256;
 }
 
-extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 8ll * (experts / 8 + 2) + 2ll * experts; }
+extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 2ll * experts + 1; }
 
 static int sorting_impl(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
                         int experts, int block_size, const int32_t* expert_mask,

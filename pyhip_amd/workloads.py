@@ -109,3 +109,17 @@ def algorithmic_work(shape, tokens, topk_ids):
                 flops_stage1=4.0 * tokens * k * I * H, flops_stage2=2.0 * tokens * k * I * H,
                 bytes_stage1=e_hit * 2.0 * I * H * (0.5 + 1.0 / 32) + tokens * H * (0.5 + 1.0 / 32),
                 bytes_stage2=e_hit * 1.0 * I * H * (0.5 + 1.0 / 32) + tokens * k * I * (0.5 + 1.0 / 32))
+
+
+def xcd_tile_counts(shape, topk_ids, block_m, pad=0):
+    """gate_up tiles per XCD for a routing: under the grouped GEMMs' schedule (the list expert -> weight tile -> row
+    block cut into 8 equal runs) and, for comparison, with whole experts dealt to the XCDs round-robin (e % 8)"""
+    cfg = SHAPES[shape] if isinstance(shape, str) else shape
+    cnt = torch.bincount(topk_ids.flatten().long().clamp(0, cfg["E"] - 1), minlength=cfg["E"]).cpu()
+    nb = (cnt + block_m - 1) // block_m
+    n_tiles = (cfg["I"] + pad + 127) // 128
+    total = int(nb.sum()) * n_tiles
+    chunk = (total + 7) // 8
+    return dict(equal_runs=[min(chunk, max(0, total - x * chunk)) for x in range(8)],
+                experts_round_robin=[int(nb[x::8].sum()) * n_tiles for x in range(8)],
+                rows_per_expert_max=int(cnt.max()), rows_per_expert_median=int(cnt.median()))

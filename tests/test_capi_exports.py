@@ -34,7 +34,7 @@ def test_size_helpers():
     assert lib.pyhip_moe_act_scale_stride(7168) == 224 and lib.pyhip_moe_act_scale_stride(1024) == 32
     assert lib.pyhip_moe_act_scale_stride(2880) == 96
     assert lib.pyhip_moe_sorting_workspace_bytes(16, 8, 256) >= 0
-    assert lib.pyhip_moe_schedule_words(256) == 8 * 34 + 512
+    assert lib.pyhip_moe_schedule_words(256) == 513
 
 
 def test_argument_errors_are_reported():
