@@ -72,6 +72,29 @@ __device__ __forceinline__ void mfma_fp4_fixed(v4i w, v4i a, int w_scale, int a_
                  : "n"(ACC0), "n"(ACC0 + 3), "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1),
                    "n"(OPW >> 1), "n"(OPA >> 1));
 }
+// The four MFMAs of one activation row group (16 rows) against the wave's four weight row groups, one assembly
+// statement.  accumulator of (weight row group j, row group mt): a[(j*MT + mt)*4 .. +3]; scale bytes: see mfma_fp4.
+// (Row groups that hold only padding are NOT skipped.  Measured with a compare and a branch around the four MFMAs
+// inside this statement, so that nothing else about the generated code changes: the pair costs more issue time in
+// full tiles than the skipped MFMAs save elsewhere: DeepSeek-V3 shape, 8192 tokens, where a fifth of the row groups
+// are padding: gate_up 1.30 -> 1.38 ms; Mixtral shape, 4096 tokens, no padding: 0.477 -> 0.503 ms.)
+template <int U, int MTI, int MT>
+__device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale)
+{
+    constexpr int A0 = (0 * MT + MTI) * 4, A1 = (1 * MT + MTI) * 4, A2 = (2 * MT + MTI) * 4, A3 = (3 * MT + MTI) * 4;
+    constexpr int W0 = (U & 1) * 2 + 0, W1 = (U & 1) * 2 + 1;       // weight-scale byte: (kt%2)*2 + (row%32)/16
+#define MFMA_TEXT(ACC, ACCE, W, WS, WL, WH)                                                                            \
+    "v_mfma_scale_f32_16x16x128_f8f6f4 a[%[" #ACC "]:%[" #ACCE "]], %[" #W "], %[a], a[%[" #ACC "]:%[" #ACCE "]], %[" #WS  \
+    "], %[as] op_sel:[%[" #WL "],%[al],0] op_sel_hi:[%[" #WH "],%[ah],0] cbsz:4 blgp:4\n\t"
+    asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
+                 MFMA_TEXT(c2, e2, w2, s23, x0l, x0h) MFMA_TEXT(c3, e3, w3, s23, x1l, x1h)
+                 :
+                 : [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3), [c2] "n"(A2), [e2] "n"(A2 + 3),
+                   [c3] "n"(A3), [e3] "n"(A3 + 3), [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
+                   [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [x0l] "n"(W0 & 1), [x0h] "n"(W0 >> 1),
+                   [x1l] "n"(W1 & 1), [x1h] "n"(W1 >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
+#undef MFMA_TEXT
+}
 template <int R>
 __device__ __forceinline__ float acc_fixed_read()
 {
@@ -201,7 +224,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // The accumulators live in the accumulation registers a0 .. a[16*MT-1], named by hand in the instruction text
     // (mfma_fp4_fixed); the clobber reserves that range for the kernel.  RING: the one-wave-per-SIMD 256-row tile
     // reads its LDS operands through a deeper ring of registers.
-    constexpr bool RING = MT > 8;
+    constexpr bool RING = true;
     if constexpr(MT == 16) asm volatile("" ::: "a0", "a255");
     if constexpr(MT == 8) asm volatile("" ::: "a0", "a127");
     if constexpr(MT == 4) asm volatile("" ::: "a0", "a63");
@@ -357,11 +380,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // Row groups of a tile that hold at least one real row.  The sort pads every expert's rows at the END of
     // its last block, so the real rows of a block are a prefix.  Padded rows send their activation fetches out
     // of the descriptor's range, where the hardware drops them, and the epilogue leaves padded row groups out.
-    // Their MFMAs are still issued: the K-group body exists once.  (Instantiating it per count of active row
-    // groups and branching between the instances is NOT safe with this pipeline: the register allocator then
-    // gives the weight-tile registers different homes in different instances and copies them at the joins,
-    // while loads into them are still in flight, which it cannot know.  Measured: wrong results in tiles that
-    // run short K-groups.  tests/test_build_checks.py looks for such copies in the generated code.)
+    // Their MFMAs are still issued: the K-group body exists once (see mfma_row_group for what skipping them costs).
+    // (Instantiating the body per count of active row groups and branching between the instances in C++ is NOT safe
+    // with this pipeline: the register allocator then gives the weight-tile registers different homes in different
+    // instances and copies them at the joins, while loads into them are still in flight, which it cannot know.
+    // Measured: wrong results in tiles that run short K-groups.  tests/test_build_checks.py looks for such copies in
+    // the generated code.)
     constexpr u32 OOB = 0xFFFF0000u;               // beyond every activation buffer (checked by the launcher)
     auto count_groups = [&](const u32* ids) __attribute__((always_inline)) -> int {
         const u32 id  = ids[(lane < MT ? lane : 0) * 16];
@@ -646,7 +670,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         // MFMAs, prefetches and weight loads of the K-group
         constexpr int MA  = MT;                   // row groups that take part
         constexpr int PPM = (NPF + MA - 1) / MA;  // prefetch operations issued after each row group's MFMAs
-        constexpr int RA = 4;
+        constexpr int RA = MT > 8 ? 4 : 2;
         v4i af_r[RA + 1];
         int asc_all[RING ? MT : 1];              // the scale dword of a row group serves all four K-steps
         auto lds_read = [&](auto NN) __attribute__((always_inline)) {
@@ -700,13 +724,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                     asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                {
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                mfma_fp4_fixed<(u & 1) * 2 + 0, u, (0 * MT + mt) * 4>(wf[u][0], af, w_sc[p][0 + (u >> 1)], asc);
-                mfma_fp4_fixed<(u & 1) * 2 + 1, u, (1 * MT + mt) * 4>(wf[u][1], af, w_sc[p][0 + (u >> 1)], asc);
-                mfma_fp4_fixed<(u & 1) * 2 + 0, u, (2 * MT + mt) * 4>(wf[u][2], af, w_sc[p][2 + (u >> 1)], asc);
-                mfma_fp4_fixed<(u & 1) * 2 + 1, u, (3 * MT + mt) * 4>(wf[u][3], af, w_sc[p][2 + (u >> 1)], asc);
-                }
+                mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
+                                          w_sc[p][2 + (u >> 1)], asc);
                 // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
                 // issue overlaps the matrix pipeline instead of preceding it
                 if constexpr(u == 0)
