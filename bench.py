@@ -12,7 +12,8 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
                roofline fractions.  Layers whose weights fit the 256 MB last-level cache rotate over
                several copies of the weights, as the reference's harness does (src/misc.py:180-273)
   decode       the headline shape at --decode-tokens (default 16), the HBM-bound end of the metric, with the
-               same call captured in a HIP graph and replayed
+               same call captured in a HIP graph and replayed; decode_other_method: the kernel family "auto" did
+               not pick, forced
   roofline     the dominant kernel (stage-1 gate_up GEMM) of the headline workload: average launch duration
                from HIP events recorded on the launch stream around that launch in a separate, untimed pass
                of the step-by-step path; traffic is read from the committed counter summary under profiles/
@@ -283,7 +284,8 @@ def main():
             main_stage = stage_pass(torch, fused_moe, W, main_res, a.block_m, a.method)
             dec = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m)
             dec_stage = stage_pass(torch, fused_moe, W, dec, a.block_m, "auto")
-            dec4 = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, "a4w4")
+            other = "a4w4" if dec["method"] == "w4a16" else "w4a16"
+            dec4 = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, other)
             dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
             cpu = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds) if a.cpu_seconds > 0 else None
         del W
@@ -334,12 +336,13 @@ def main():
                    "tflops": round(dw["flops"] / (dec["median_ms"] * 1e-3) / 1e12, 2),
                    "stage_ms_untimed_pass": {k: round(v, 4) for k, v in dec_stage.items()},
                    "graph_replay_ms_per_step": round(dec_graph_ms, 4),
-                   "roofline": {"kernel": "moe_gemm_w4a16_kernel<1,1> (gate_up, bf16 activations)", "bound": "hbm",
+                   "roofline": {"kernel": "moe_gemm_w4a16_kernel<1,1> (gate_up, bf16 activations)" if dec["method"] == "w4a16"
+                                else "moe_gemm_mxfp4_kernel<1,1,0,true> (gate_up, MXFP4 activations)", "bound": "hbm",
                                 "achieved": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBPS,
                                 "unit": "GB/s",
                                 "frac": round(dw["bytes_stage1"] / (dg1_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                                 "traffic": dtraffic, "avg_launch_ms": round(dg1_ms, 4)}},
-        "decode_a4w4": {"tokens": a.decode_tokens, "ms_per_step": round(dec4["median_ms"], 4),
+        "decode_other_method": {"tokens": a.decode_tokens, "method": dec4["method"], "ms_per_step": round(dec4["median_ms"], 4),
                         "hbm_gbps": round(dw["bytes"] / (dec4["median_ms"] * 1e-3) / 1e9, 1),
                         "frac_of_hbm_peak": round(dw["bytes"] / (dec4["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)},
         "configs": configs,

@@ -85,6 +85,22 @@ int pyhip_moe_sorting_quant(const int32_t* topk_ids, const float* topk_weights, 
                             const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K, uint8_t* q,
                             uint8_t* scales, pyhip_stream_t stream);
 
+/* Router + sort in one call, the two steps before the GEMMs (aiter.fused_topk followed by
+ * aiter.fused_moe.moe_sorting in the reference: tests/contrib/moe/test_fused_moe.py:38,87 and
+ * src/contrib/fused_moe.py:283).  gating f32 [tokens, experts]; n_group = 0 selects pyhip_moe_topk_softmax's
+ * router, n_group > 0 pyhip_moe_topk_grouped_sigmoid's; the picks are written to topk_weight / topk_ids (both
+ * required: the top-k reduction and the caller read them) and sorted as pyhip_moe_sorting does.  x_bf16 (may be
+ * NULL) .. scales: the input quantisation of pyhip_moe_sorting_quant.  Up to 64 tokens (and 512 experts, a power of
+ * two times 64) all of it is ONE launch: the sort's single workgroup routes the tokens itself; larger inputs take
+ * the router's own launch first.  Same results either way.  experts must be a multiple of 64. */
+int pyhip_moe_route_sorting(const float* gating, int tokens, int topk, int experts, int n_group, int topk_group,
+                            int renormalize, int block_size, const int32_t* expert_mask,
+                            const int32_t* num_local_tokens, float* topk_weight, int32_t* topk_ids,
+                            uint32_t* sorted_ids, float* sorted_weights, uint32_t* sorted_expert_ids,
+                            uint32_t* num_valid_ids, uint32_t* schedule, void* workspace, int64_t workspace_bytes,
+                            const void* x_bf16, int64_t row_stride_elems, int64_t rows, int K, uint8_t* q,
+                            uint8_t* scales, pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Dynamic MXFP4 quantisation of bf16 activations (1x32 blocks, e8m0 scale
  * 2^(floor(log2 amax) - 2), e2m1 round-to-nearest-even).  Replaces
@@ -205,6 +221,18 @@ int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const 
                       const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk, int experts,
                       int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
                       void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
+
+/* pyhip_moe_forward with the router inside the call: gating f32 [tokens, experts] in (n_group / topk_group /
+ * renormalize as for pyhip_moe_route_sorting), the picks out in topk_ids / topk_weights next to the layer output.
+ * The reference's callers run aiter.fused_topk and then fused_moe (tests/contrib/moe/test_fused_moe.py:38-60). */
+int pyhip_moe_forward_routed(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
+                             const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                             const void* bias1_bf16, const void* bias2_bf16, const float* gating, int n_group,
+                             int topk_group, int renormalize, int32_t* topk_ids, float* topk_weights,
+                             const int32_t* expert_mask, const int32_t* num_local_tokens, void* out, int out_is_f32,
+                             int tokens, int topk, int experts, int hidden, int inter, int block_m, int w4a16,
+                             int split_k, int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
+                             pyhip_stream_t stream);
 
 /* pyhip_moe_forward without the workspace argument: the intermediates live in a device array that belongs to the
  * library (64 MiB, pyhip_moe_forward_static_capacity(); one copy per GPU, held until the process ends).  It has no

@@ -27,6 +27,10 @@ SIGNATURES = {
     "pyhip_moe_forward_workspace_bytes": (_L, [_L, _I, _I, _I, _I, _I, _I]),
     "pyhip_moe_forward": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                _I, _F, _P, _L, _P]),
+    "pyhip_moe_route_sorting": (_I, [_P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _L, _I,
+                                     _P, _P, _P]),
+    "pyhip_moe_forward_routed": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I,
+                                      _I, _I, _I, _I, _I, _I, _F, _P, _L, _P]),
     "pyhip_moe_forward_static_capacity": (_L, []),
     "pyhip_moe_forward_static": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                       _I, _F, _P]),

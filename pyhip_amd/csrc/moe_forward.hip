@@ -24,6 +24,9 @@ int pyhip_moe_gemm1_w4a16(const void*, const uint8_t*, const uint8_t*, const voi
                           const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, int, float, hipStream_t);
 int pyhip_moe_gemm2_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const float*,
                           const uint32_t*, const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, hipStream_t);
+int pyhip_moe_route_sorting(const float*, int, int, int, int, int, int, int, const int32_t*, const int32_t*, float*, int32_t*,
+                            uint32_t*, float*, uint32_t*, uint32_t*, uint32_t*, void*, int64_t, const void*, int64_t, int64_t,
+                            int, uint8_t*, uint8_t*, hipStream_t);
 int pyhip_moe_topk_reduce_routed(const void*, void*, int64_t, int, int, int, const int32_t*, int, const int32_t*,
                                  const int32_t*, hipStream_t);
 }
@@ -87,8 +90,14 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
 
 extern "C" int pyhip_moe_pick_w4a16(int64_t tokens, int topk, int experts, int hidden)
 {
+    // bf16 activations win (a) when at most one expert in eight gets a row at all (DeepSeek-V3 shape: 1 token 0.046
+    // against 0.051 ms, 4 tokens 0.128 against 0.127 ms, 16 tokens 0.393 against 0.377 ms; gpt-oss shape: 4 tokens 0.053
+    // against 0.055 ms, 16 tokens 0.141 against 0.134 ms), and (b) in layers with so few experts that the down GEMM of
+    // the MXFP4-activation path has fewer than 512 tiles, which the bf16 kernel splits K-wise over four times as many
+    // workgroups (Mixtral shape: 1 token 0.054 against 0.071 ms, 16 tokens 0.132 against 0.137 ms, 64 tokens 0.181
+    // against 0.140 ms)
     const int64_t pairs  = tokens * topk;
-    const bool sparse    = 4 * pairs <= 3 * (int64_t)experts;
+    const bool sparse    = 8 * pairs <= (int64_t)experts;
     const bool few_tiles = (pairs < experts ? pairs : experts) * (hidden / 256) < 512 && pairs <= 8 * (int64_t)experts;
     return sparse || few_tiles;
 }
@@ -101,14 +110,20 @@ extern "C" int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, i
     return make_layout(tokens, topk, experts, hidden, inter, block_m, w4a16).total;
 }
 
-extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
-                                 const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
-                                 const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
-                                 const float* topk_weights, const int32_t* expert_mask,
-                                 const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk,
-                                 int experts, int hidden, int inter, int block_m, int w4a16, int split_k,
-                                 int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
-                                 hipStream_t stream)
+namespace {
+struct Router
+{
+    const float* gating = nullptr;      // [tokens, experts] or null: topk_ids / topk_weights are inputs
+    int n_group = 0, topk_group = 0, renormalize = 1;
+};
+}   // namespace
+
+static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1, const uint8_t* w1_scale,
+                        const uint8_t* w2, const uint8_t* w2_scale, const void* bias1_bf16, const void* bias2_bf16,
+                        const Router& router, int32_t* topk_ids, float* topk_weights, const int32_t* expert_mask,
+                        const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk, int experts,
+                        int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
+                        void* workspace, int64_t workspace_bytes, hipStream_t stream)
 {
     PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && w2 && w2_scale && topk_ids && topk_weights && out,
                   "moe_forward: null pointer");
@@ -128,7 +143,14 @@ extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_str
     uint32_t* sched   = (uint32_t*)(ws + l.sched);
     void* out3        = ws + l.out3;
     int rc;
-    if(w4a16)
+    if(router.gating)
+        // the routing is part of the call: the sort's own workgroup routes the tokens when there are few of them
+        rc = pyhip_moe_route_sorting(router.gating, tokens, topk, experts, router.n_group, router.topk_group,
+                                     router.renormalize, block_m, expert_mask, num_local_tokens, topk_weights, topk_ids,
+                                     s_ids, s_w, s_e, n_valid, sched, ws + l.sort_ws, l.sort_ws_bytes,
+                                     w4a16 ? nullptr : hidden_bf16, hidden_row_stride, tokens, hidden,
+                                     w4a16 ? nullptr : ws + l.a1_q, w4a16 ? nullptr : ws + l.a1_s, stream);
+    else if(w4a16)
         rc = pyhip_moe_sorting(topk_ids, topk_weights, tokens, topk, experts, block_m, expert_mask, num_local_tokens,
                                s_ids, s_w, s_e, n_valid, sched, nullptr, 0, ws + l.sort_ws, l.sort_ws_bytes, stream);
     else
@@ -163,4 +185,38 @@ extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_str
     // clearing and the traffic under expert parallelism is that of the owned slots.
     return pyhip_moe_topk_reduce_routed(out3, out, tokens, topk, hidden, out_is_f32, topk_ids, experts, expert_mask,
                                         num_local_tokens, stream);
+}
+
+extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
+                                 const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                                 const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
+                                 const float* topk_weights, const int32_t* expert_mask,
+                                 const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk,
+                                 int experts, int hidden, int inter, int block_m, int w4a16, int split_k,
+                                 int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
+                                 hipStream_t stream)
+{
+    return forward_impl(hidden_bf16, hidden_row_stride, w1, w1_scale, w2, w2_scale, bias1_bf16, bias2_bf16, Router{},
+                        const_cast<int32_t*>(topk_ids), const_cast<float*>(topk_weights), expert_mask, num_local_tokens,
+                        out, out_is_f32, tokens, topk, experts, hidden, inter, block_m, w4a16, split_k, activation,
+                        swiglu_limit, workspace, workspace_bytes, stream);
+}
+
+// The layer with its router: gating scores in, and the picks (topk_ids, topk_weights) out next to the layer output.
+// n_group = 0: softmax over the experts, top-k; n_group > 0: sigmoid scores with grouped selection (DeepSeek-V3).
+extern "C" int pyhip_moe_forward_routed(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
+                                        const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                                        const void* bias1_bf16, const void* bias2_bf16, const float* gating, int n_group,
+                                        int topk_group, int renormalize, int32_t* topk_ids, float* topk_weights,
+                                        const int32_t* expert_mask, const int32_t* num_local_tokens, void* out,
+                                        int out_is_f32, int tokens, int topk, int experts, int hidden, int inter,
+                                        int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
+                                        void* workspace, int64_t workspace_bytes, hipStream_t stream)
+{
+    PYHIP_REQUIRE(gating, "moe_forward_routed: null gating scores");
+    Router r;
+    r.gating = gating; r.n_group = n_group; r.topk_group = topk_group; r.renormalize = renormalize;
+    return forward_impl(hidden_bf16, hidden_row_stride, w1, w1_scale, w2, w2_scale, bias1_bf16, bias2_bf16, r, topk_ids,
+                        topk_weights, expert_mask, num_local_tokens, out, out_is_f32, tokens, topk, experts, hidden, inter,
+                        block_m, w4a16, split_k, activation, swiglu_limit, workspace, workspace_bytes, stream);
 }

@@ -809,10 +809,11 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
                              // schedule table in LDS holds: one tile per workgroup
     if(g.sched)
     {
-        // persistent: two workgroups per CU (one for 256-row tiles).  Small tiles would fit three or four; measured,
-        // that changes nothing: they are bound by the weight stream
+        // persistent: as many workgroups per CU as fit (three of the 16- and 32-row tiles, two up to 128 rows, one of
+        // the 256-row tile).  The small tiles are bound by the weight stream; what the third workgroup buys is fewer,
+        // fuller rounds when the tiles number little more than the resident workgroups
         const int cus = device_cu_count();
-        unsigned resident = (unsigned)cus * (block_m <= 128 ? 2u : 1u) / 8u * 8u;
+        unsigned resident = (unsigned)cus * (block_m <= 32 ? 3u : block_m <= 128 ? 2u : 1u) / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
     }
     dim3 grid(nwg), block(GEMM_THREADS);

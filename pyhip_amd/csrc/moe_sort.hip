@@ -15,6 +15,7 @@
 // launch for small inputs.
 #include "common.h"
 #include "quant_device.h"
+#include "router_device.h"
 
 #define SORT_THREADS 256
 #define SORT_WAVES (SORT_THREADS / WAVE)
@@ -37,6 +38,16 @@ struct SortArgs
     u32* ws;                   // workspace: hist[G][E], then per-expert offset[E]
     u32* sched;                // optional tile schedule for the grouped GEMMs (see write_schedule) or null
     int T_all, k, E, Bm, n_blk, G;
+};
+
+// routing done by the sort's own workgroup (single-workgroup sort only): gating scores in, the top-k picks written
+// to the buffers the sort then reads its pairs from
+struct RouteArgs
+{
+    const float* gating;       // [T_all, E] (E = 64 * NE) or null: the pairs are given
+    float* topk_w;             // [T_all, k] out
+    int* topk_ids;             // [T_all, k] out
+    int n_group, topk_group, renorm;
 };
 
 __device__ __forceinline__ int sort_tokens(const SortArgs& a)
@@ -277,7 +288,10 @@ __device__ __forceinline__ void write_schedule(const SortArgs& a, const u32* off
 // LDS: whist[SMALL_WAVES][E] | tot[E] | off[E] | lid[E] | scratch[2*SMALL_WAVES]
 // Workgroups past the first quantise activations (qa.rows > 0): the input quantisation of the MXFP4-activation
 // path depends on nothing the sort computes, and carrying it in this launch saves a dispatch.
-extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a, QuantArgs qa)
+// NE > 0: the workgroup first routes the tokens itself (a wave per token, tokens dealt round-robin to its 16 waves;
+// the step before the sort, aiter.fused_topk at tests/contrib/moe/test_fused_moe.py:38,87, costs no launch of its own).
+template <int NE, bool GROUPED>
+__global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kernel(SortArgs a, QuantArgs qa, RouteArgs ra)
 {
     if(blockIdx.x > 0)
     {
@@ -295,6 +309,26 @@ extern "C" __global__ void __launch_bounds__(SMALL_THREADS) moe_sort_small_kerne
     const int wave  = threadIdx.x / WAVE;
     const int cv    = wave_chunk(pairs, SMALL_WAVES);
     const int beg   = min(pairs, wave * cv), end = min(pairs, beg + cv);
+
+    if constexpr(NE > 0)
+    {
+        const int lane = lane_id();
+        for(int t = wave; t < a.T_all; t += SMALL_WAVES)
+        {
+            float w;
+            int id;
+            route_token<NE, GROUPED>(ra.gating + (size_t)t * a.E, lane, a.k, ra.n_group, ra.topk_group, ra.renorm, w, id);
+            if(lane < a.k)
+            {
+                ra.topk_w[(size_t)t * a.k + lane]   = w;
+                ra.topk_ids[(size_t)t * a.k + lane] = id;
+            }
+        }
+        // the picks reach the L2 before any wave of this workgroup reads them back as the sort's pairs (these
+        // addresses have not been read by this kernel before, so no stale line can sit in the CU's cache)
+        __threadfence();
+        __syncthreads();
+    }
 
     WavePairs<SMALL_GROUPS> wp;
     wp.load(a, beg, end, true);
@@ -500,12 +534,37 @@ extern "C" int64_t pyhip_moe_sorting_workspace_bytes(int64_t tokens, int topk, i
 
 extern "C" int64_t pyhip_moe_schedule_words(int experts) { return 2ll * experts + 1; }
 
+// most tokens / experts the single-workgroup sort routes itself; beyond, the router gets a launch of its own
+#define ROUTE_SORT_MAX_TOKENS 64
+#define ROUTE_SORT_MAX_EXPERTS 512
+
+static int launch_routing_sort(const SortArgs& a, const QuantArgs& qa, const RouteArgs& ra, unsigned qblocks, size_t lds,
+                               hipStream_t stream)
+{
+    const dim3 grid(1 + qblocks), block(SMALL_THREADS);
+#define ROUTE_SORT_CASE(N)                                                                                            \
+    case N:                                                                                                           \
+        if(ra.n_group > 0)                                                                                            \
+            hipLaunchKernelGGL((moe_sort_small_kernel<N, true>), grid, block, lds, stream, a, qa, ra);                \
+        else                                                                                                          \
+            hipLaunchKernelGGL((moe_sort_small_kernel<N, false>), grid, block, lds, stream, a, qa, ra);               \
+        break;
+    switch(a.E / 64)
+    {
+        ROUTE_SORT_CASE(1) ROUTE_SORT_CASE(2) ROUTE_SORT_CASE(4) ROUTE_SORT_CASE(8)
+    default: pyhip_set_error("moe_route_sorting: experts/64 = %d not in {1,2,4,8}", a.E / 64); return PYHIP_ERR_INVALID;
+    }
+#undef ROUTE_SORT_CASE
+    PYHIP_CHECK_LAUNCH("moe_sort_small_kernel (routing)");
+    return PYHIP_OK;
+}
+
 static int sorting_impl(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
                         int experts, int block_size, const int32_t* expert_mask,
                         const int32_t* num_local_tokens, uint32_t* sorted_ids, float* sorted_weights,
                         uint32_t* sorted_expert_ids, uint32_t* num_valid_ids, uint32_t* schedule,
                         void* moe_out, int64_t moe_out_bytes, void* workspace, int64_t workspace_bytes,
-                        QuantArgs qa, hipStream_t stream)
+                        QuantArgs qa, RouteArgs ra, hipStream_t stream)
 {
     PYHIP_REQUIRE(topk_ids && topk_weights && sorted_ids && sorted_weights && sorted_expert_ids && num_valid_ids,
                   "moe_sorting: null pointer");
@@ -555,11 +614,14 @@ static int sorting_impl(const int32_t* topk_ids, const float* topk_weights, int 
         size_t lds = ((size_t)(SMALL_WAVES + 3) * experts + 2 * SMALL_WAVES + 2) * 4;
         if(lds > 64 * 1024)
         {
-            hipError_t e = hipFuncSetAttribute((const void*)moe_sort_small_kernel,
+            PYHIP_REQUIRE(!ra.gating, "moe_sorting: the routing sort handles at most %d experts", ROUTE_SORT_MAX_EXPERTS);
+            hipError_t e = hipFuncSetAttribute((const void*)moe_sort_small_kernel<0, false>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             PYHIP_REQUIRE(e == hipSuccess, "moe_sorting: cannot reserve %zu B of LDS", lds);
         }
-        hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1 + qblocks), dim3(SMALL_THREADS), lds, stream, a, qa);
+        if(ra.gating)
+            return launch_routing_sort(a, qa, ra, qblocks, lds, stream);
+        hipLaunchKernelGGL((moe_sort_small_kernel<0, false>), dim3(1 + qblocks), dim3(SMALL_THREADS), lds, stream, a, qa, ra);
         PYHIP_CHECK_LAUNCH("moe_sort_small_kernel");
         return PYHIP_OK;
     }
@@ -585,7 +647,7 @@ extern "C" int pyhip_moe_sorting(const int32_t* topk_ids, const float* topk_weig
     QuantArgs qa = {};
     return sorting_impl(topk_ids, topk_weights, tokens, topk, experts, block_size, expert_mask, num_local_tokens,
                         sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, schedule, moe_out, moe_out_bytes,
-                        workspace, workspace_bytes, qa, stream);
+                        workspace, workspace_bytes, qa, RouteArgs{}, stream);
 }
 
 extern "C" int pyhip_moe_sorting_quant(const int32_t* topk_ids, const float* topk_weights, int tokens, int topk,
@@ -602,5 +664,57 @@ extern "C" int pyhip_moe_sorting_quant(const int32_t* topk_ids, const float* top
         return rc;
     return sorting_impl(topk_ids, topk_weights, tokens, topk, experts, block_size, expert_mask, num_local_tokens,
                         sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, schedule, nullptr, 0, workspace,
-                        workspace_bytes, qa, stream);
+                        workspace_bytes, qa, RouteArgs{}, stream);
+}
+
+int pyhip_check_router(const char* name, const void* logits, const void* w, const void* ids, int tokens, int experts,
+                       int topk);
+extern "C" int pyhip_moe_topk_softmax(const float*, int, int, int, int, float*, int32_t*, hipStream_t);
+extern "C" int pyhip_moe_topk_grouped_sigmoid(const float*, int, int, int, int, int, int, float*, int32_t*, hipStream_t);
+
+// Router + sort (+ optional input quantisation).  Up to ROUTE_SORT_MAX_TOKENS tokens (and pairs that fit the
+// single-workgroup sort) everything is ONE launch: the sort's workgroup routes the tokens itself.  Larger inputs take
+// the router's own launch followed by the sort; the results are the same either way.
+extern "C" int pyhip_moe_route_sorting(const float* gating, int tokens, int topk, int experts, int n_group,
+                                       int topk_group, int renormalize, int block_size, const int32_t* expert_mask,
+                                       const int32_t* num_local_tokens, float* topk_weight, int32_t* topk_ids,
+                                       uint32_t* sorted_ids, float* sorted_weights, uint32_t* sorted_expert_ids,
+                                       uint32_t* num_valid_ids, uint32_t* schedule, void* workspace,
+                                       int64_t workspace_bytes, const void* x_bf16, int64_t row_stride_elems,
+                                       int64_t rows, int K, uint8_t* q, uint8_t* scales, hipStream_t stream)
+{
+    int rc = pyhip_check_router("moe_route_sorting", gating, topk_weight, topk_ids, tokens, experts, topk);
+    if(rc)
+        return rc;
+    PYHIP_REQUIRE(n_group >= 0 && (n_group == 0 || (n_group <= 64 && (n_group & (n_group - 1)) == 0 &&
+                                                   experts % n_group == 0 && topk_group >= 1 && topk_group <= n_group &&
+                                                   topk <= topk_group * (experts / n_group))),
+                  "moe_route_sorting: n_group=%d topk_group=%d (0 groups = softmax router)", n_group, topk_group);
+    QuantArgs qa = {};
+    if(x_bf16)
+    {
+        rc = pyhip_make_quant_args("moe_route_sorting", x_bf16, row_stride_elems, rows, K, q, scales, nullptr, &qa);
+        if(rc)
+            return rc;
+    }
+    RouteArgs ra  = {};
+    const int ne  = experts / 64;
+    const bool fused = tokens > 0 && tokens <= ROUTE_SORT_MAX_TOKENS && (int64_t)tokens * topk <= SMALL_PAIRS_MAX &&
+                       experts <= ROUTE_SORT_MAX_EXPERTS && (ne & (ne - 1)) == 0;
+    if(fused)
+    {
+        ra.gating = gating; ra.topk_w = topk_weight; ra.topk_ids = topk_ids;
+        ra.n_group = n_group; ra.topk_group = topk_group; ra.renorm = renormalize;
+    }
+    else
+    {
+        rc = n_group > 0 ? pyhip_moe_topk_grouped_sigmoid(gating, tokens, experts, topk, n_group, topk_group, renormalize,
+                                                          topk_weight, topk_ids, stream)
+                         : pyhip_moe_topk_softmax(gating, tokens, experts, topk, renormalize, topk_weight, topk_ids, stream);
+        if(rc)
+            return rc;
+    }
+    return sorting_impl(topk_ids, topk_weight, tokens, topk, experts, block_size, expert_mask, num_local_tokens,
+                        sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, schedule, nullptr, 0, workspace,
+                        workspace_bytes, qa, ra, stream);
 }

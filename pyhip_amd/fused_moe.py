@@ -11,8 +11,7 @@ Pipeline (all launches on the current torch stream, no host synchronisation):
 
 ``method="w4a16"`` keeps the activations in bf16 (weights are expanded to bf16 in registers), the variant the
 reference runs for few tokens (src/contrib/moe.py:362-787); ``method="a4w4"`` forces the MXFP4-activation path;
-``method="auto"`` takes w4a16 up to 2 routed rows per expert on average (where it is the faster of the two on
-MI355X and the layer is bound by weight streaming) and a4w4 above.
+``method="auto"`` takes w4a16 for the very smallest calls (see ``pick_w4a16``) and a4w4 above.
 """
 import torch
 
@@ -20,7 +19,7 @@ from . import _lib
 from .enums import ActivationType, QuantType
 from .moe_sorting import moe_sorting, max_blocks
 
-__all__ = ["fused_moe"]
+__all__ = ["fused_moe", "fused_moe_routed"]
 
 
 def _as_u8(t):
@@ -84,11 +83,10 @@ def pick_block_m(tokens, topk, experts, hidden=0):
 def pick_w4a16(tokens, topk, experts, hidden):
     """``method="auto"``: True selects the bf16-activation kernels (the reference switches to its w4a16 split-K
     kernel for few tokens, src/contrib/moe.py:362-787).  They win in two regimes (measured on all five benchmark
-    shapes): fewer than 0.75 routed rows per expert on average (DS-V3 T = 16: 0.40 against 0.42 ms; from one row per
-    expert on the MXFP4-activation kernels stream faster), and layers with so few experts that the down GEMM of the
-    MXFP4-activation path, one workgroup per (row block, 256 output channels), cannot fill the GPU while the
-    bf16-activation kernel splits K over four times as many workgroups (Mixtral shape up to 8 rows per expert,
-    T = 1: 0.068 against 0.109 ms)."""
+    shapes, quoted next to the rule in pyhip_moe_pick_w4a16): when at most one expert in eight gets a row at all
+    (DeepSeek-V3 shape up to 4 tokens), and in layers with so few experts that the down GEMM of the MXFP4-activation
+    path, one workgroup per (row block, 256 output channels), cannot fill the GPU while the bf16-activation kernel
+    splits K over four times as many workgroups (Mixtral shape up to 32 tokens)."""
     return bool(_lib.load().pyhip_moe_pick_w4a16(tokens, topk, experts, hidden))
 
 
@@ -305,3 +303,59 @@ def fused_moe(
                          num_valid_ids=num_valid, a1_q=a1_q, a1_s=a1_s, a2=a2, a2_q=a2_q, a2_s=a2_s,
                          out3=out3, block_m=bm)
     return out
+
+
+def fused_moe_routed(hidden_states, w1, w2, gating_output, topk, renormalize=True, num_expert_group=0, topk_group=0,
+                     w1_scale=None, w2_scale=None, expert_mask=None, activation=ActivationType.Silu,
+                     block_size_M=None, num_local_tokens=None, dtype=None, bias1=None, bias2=None, splitk=0,
+                     method="auto", swiglu_limit=None, return_routing=False):
+    """``fused_topk`` (or ``grouped_topk`` when ``num_expert_group > 0``) followed by ``fused_moe``, as the reference's
+    callers chain them (tests/contrib/moe/test_fused_moe.py:38-60), in one library call: for up to 64 tokens the
+    router runs inside the sort's launch.  ``gating_output`` f32 [T, E], E a multiple of 64 (use ``fused_topk`` +
+    ``fused_moe`` otherwise).  -> out, or (out, topk_weights, topk_ids) with ``return_routing``."""
+    lib = _lib.load()
+    _require(activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts only")
+    act = 1 if activation == ActivationType.Swiglu else 0
+    limit = float(swiglu_limit) if swiglu_limit else 7.0
+    _require(w1_scale is not None and w2_scale is not None, "w1_scale and w2_scale (e8m0, shuffled) are required")
+    _require(hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2,
+             "hidden_states must be a bf16 matrix on the GPU", TypeError)
+    out_dtype = hidden_states.dtype if dtype is None else dtype
+    _require(out_dtype in (torch.bfloat16, torch.float32), "dtype must be bfloat16 or float32", TypeError)
+    _require(method in ("auto", "a4w4", "w4a16"), "method=%r" % (method,))
+    w1u, w2u, w1s, w2s = _shuffled_u8(w1), _shuffled_u8(w2), _as_u8(w1_scale), _as_u8(w2_scale)
+    T, H = hidden_states.shape
+    E, N1, Hb = w1u.shape
+    I = N1 // 2
+    _require(Hb * 2 == H and tuple(w2u.shape) == (E, H, I // 2), "shapes do not fit")
+    global_E = E if expert_mask is None else expert_mask.numel()
+    _require(gating_output.is_cuda and tuple(gating_output.shape) == (T, global_E) and global_E % 64 == 0,
+             "gating_output must be [tokens, experts] on the GPU with experts a multiple of 64")
+    g = gating_output.float().contiguous()
+    dev = hidden_states.device
+    if expert_mask is not None:
+        expert_mask = expert_mask.to(device=dev, dtype=torch.int32).contiguous()
+    w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, topk, global_E, H))
+    bm = block_size_M if block_size_M is not None else pick_block_m(T, topk, global_E, H)
+    if w4a16:
+        bm = min(bm, 64)
+    if bias1 is not None:
+        bias1 = bias1.to(torch.bfloat16).contiguous()
+    if bias2 is not None:
+        bias2 = bias2.to(torch.bfloat16).contiguous()
+    x = hidden_states
+    if x.stride(1) != 1 or (w4a16 and x.stride(0) != H) or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+        x = x.contiguous()
+    ws_bytes = lib.pyhip_moe_forward_workspace_bytes(T, topk, global_E, H, I, bm, 1 if w4a16 else 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    out = torch.empty(T, H, dtype=out_dtype, device=dev)
+    tw = torch.empty(T, topk, dtype=torch.float32, device=dev)
+    ti = torch.empty(T, topk, dtype=torch.int32, device=dev)
+    rc = lib.pyhip_moe_forward_routed(_lib.dptr(x), x.stride(0), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(w2u),
+                                      _lib.dptr(w2s), _lib.dptr(bias1), _lib.dptr(bias2), _lib.dptr(g),
+                                      int(num_expert_group), int(topk_group), 1 if renormalize else 0, _lib.dptr(ti),
+                                      _lib.dptr(tw), _lib.dptr(expert_mask), _lib.dptr(num_local_tokens), _lib.dptr(out),
+                                      1 if out_dtype == torch.float32 else 0, T, topk, global_E, H, I, bm,
+                                      1 if w4a16 else 0, splitk, act, limit, _lib.dptr(ws), ws_bytes, _lib.current_stream())
+    _lib.check(rc, "moe_forward_routed")
+    return (out, tw, ti) if return_routing else out

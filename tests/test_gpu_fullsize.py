@@ -21,9 +21,9 @@ pytestmark = pytest.mark.gpu
 # MXFP4-activation family is forced as well (and the other way round at the decode sizes of DeepSeek-V3).
 CASES = {
     "mixtral": [(1, "auto"), (1, "a4w4"), (32, "auto"), (32, "a4w4"), (512, "auto"), (4096, "auto")],
-    "gptoss": [(16, "auto"), (16, "a4w4"), (256, "auto"), (4096, "auto")],
+    "gptoss": [(16, "auto"), (16, "w4a16"), (256, "auto"), (4096, "auto")],
     "qwen3": [(64, "auto"), (64, "w4a16"), (2048, "auto"), (8192, "auto")],
-    "dsv3": [(16, "auto"), (16, "a4w4"), (128, "auto"), (1024, "auto"), (8192, "auto"), (32768, "a4w4")],
+    "dsv3": [(16, "auto"), (16, "w4a16"), (128, "auto"), (1024, "auto"), (8192, "auto"), (32768, "a4w4")],
 }
 SAMPLED_EXPERTS = {"mixtral": 1, "gptoss": 2, "qwen3": 2, "dsv3": 2}
 

@@ -336,8 +336,8 @@ def test_prepared_weight_file_feeds_the_operator(tmp_path):
 
 
 def test_auto_dispatch():
-    """method="auto": bf16 activations below 0.75 routed rows per expert on average, MXFP4 activations above"""
-    L = cases.make_layer("dsv3_s", 4, seed=2)             # 4 * 8 / 64 = 0.5 rows per expert
+    """method="auto": bf16 activations for the smallest calls (see pick_w4a16), MXFP4 activations above"""
+    L = cases.make_layer("dsv3_s", 1, seed=2)             # 8 pairs over 64 experts
     w1, w1s, w2, w2s = cases.device_weights(L)
     tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
     kw = dict(w1_scale=w1s, w2_scale=w2s)

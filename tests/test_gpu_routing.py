@@ -77,3 +77,30 @@ def test_routed_layer_end_to_end():
     torch.cuda.synchronize()
     rms = b.float().pow(2).mean().sqrt().item()
     assert (a - b).abs().max().item() <= 1e-4 * rms          # only the fp32 routing weights differ
+
+
+@pytest.mark.parametrize("T,router,method", [(1, "grouped", "w4a16"), (16, "grouped", "auto"), (64, "softmax", "a4w4"),
+                                             (65, "softmax", "a4w4"), (300, "grouped", "a4w4")])
+def test_router_inside_the_layer_call(T, router, method):
+    """fused_moe_routed (router + sort + GEMMs + reduce behind one library call; up to 64 tokens the sort's own
+    workgroup routes the tokens, beyond that the router has its launch) gives, bit for bit, the picks of the
+    stand-alone router and the output of fused_moe on those picks."""
+    import cases
+    from pyhip_amd import fused_moe, fused_moe_routed
+    L = cases.make_layer("dsv3_s", T, seed=7)                          # E=64, top-8
+    g = torch.Generator().manual_seed(70 + T)
+    logits = torch.randn(T, L.E, generator=g).cuda()
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    print(f"routed-layer case T={T} router={router} method={method}", flush=True)
+    if router == "grouped":
+        w, ids = routing.grouped_topk(logits, L.k, True, 8, 4)
+        kw = dict(num_expert_group=8, topk_group=4)
+    else:
+        w, ids = routing.fused_topk(None, logits, L.k, True)
+        kw = {}
+    ref = fused_moe(L.hidden.cuda(), w1, w2, w, ids, w1_scale=w1s, w2_scale=w2s, method=method)
+    out, tw, ti = fused_moe_routed(L.hidden.cuda(), w1, w2, logits, L.k, True, w1_scale=w1s, w2_scale=w2s, method=method,
+                                   return_routing=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(ti, ids) and torch.equal(tw, w)
+    assert torch.equal(out, ref) and torch.isfinite(out.float()).all()

@@ -91,19 +91,20 @@ def test_row_block_heuristic():
 
 
 def test_auto_method_rule():
-    """bf16 activations below 0.75 routed rows per expert, or while few experts leave the down GEMM short of tiles"""
+    """bf16 activations while at most one expert in eight gets a row, or while few experts leave the down GEMM short of
+    tiles"""
     from pyhip_amd.fused_moe import pick_w4a16
-    assert pick_w4a16(16, 8, 256, 7168) and pick_w4a16(24, 8, 256, 7168)          # DS-V3: 0.5 and 0.75 rows per expert
-    assert not pick_w4a16(32, 8, 256, 7168) and not pick_w4a16(8192, 8, 256, 7168)
-    assert pick_w4a16(8, 8, 128, 4096) and not pick_w4a16(16, 8, 128, 4096)       # Qwen3
-    assert pick_w4a16(16, 4, 128, 3072) and not pick_w4a16(32, 4, 128, 3072)      # gpt-oss, padded width
+    assert pick_w4a16(1, 8, 256, 7168) and pick_w4a16(4, 8, 256, 7168)            # DS-V3: 8 and 32 pairs over 256 experts
+    assert not pick_w4a16(8, 8, 256, 7168) and not pick_w4a16(16, 8, 256, 7168) and not pick_w4a16(8192, 8, 256, 7168)
+    assert pick_w4a16(2, 8, 128, 4096) and not pick_w4a16(4, 8, 128, 4096)        # Qwen3
+    assert pick_w4a16(4, 4, 128, 3072) and not pick_w4a16(16, 4, 128, 3072)       # gpt-oss, padded width
     assert pick_w4a16(1, 2, 8, 4096) and pick_w4a16(32, 2, 8, 4096)               # Mixtral: 8 experts x 16 tiles
     assert not pick_w4a16(48, 2, 8, 4096) and not pick_w4a16(4096, 2, 8, 4096)
     assert not pick_w4a16(64, 2, 8, 1024)                                         # the tiny shape at 16 rows per expert
 
 
 def test_library_makes_the_same_choices():
-    """pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 (for callers without the Python layer) agree with the host code"""
+    """the host functions are thin calls of pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 (one source of truth)"""
     from pyhip_amd import _lib
     from pyhip_amd.fused_moe import pick_block_m, pick_w4a16
     lib = _lib.load()
