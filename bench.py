@@ -57,6 +57,8 @@ def parse():
     ap.add_argument("--block-m", type=int, default=0)
     ap.add_argument("--method", default="auto")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="target size of the CPU sample; 0 = skip")
+    ap.add_argument("--epilogue-comparison", action="store_true",
+                    help="also time the down GEMM with the atomic top-k epilogue against store + reduction")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
     return ap.parse_args()
@@ -148,6 +150,26 @@ def stage_pass(torch, fused_moe, W, res, block_m, method, passes=8):
     for name, a, b in events:
         acc.setdefault(name, []).append(a.elapsed_time(b))
     return {k: sum(v) / len(v) for k, v in acc.items()}
+
+
+def epilogue_comparison(torch, fused_moe, W, res, block_m):
+    """the tail of the layer both ways, from events in untimed passes of the step-by-step path: down GEMM storing
+    out3[T, k, H] + top-k reduction (deterministic, the product path) against output clear + down GEMM with packed
+    bf16 atomics into out[T, H] (the reference's atomic variant)"""
+    r = {}
+    for mode in ("store", "atomic"):
+        kw = call_kwargs(W, block_m, "a4w4")
+        events = []
+        for i in range(10):
+            fused_moe(res["hidden"], W["w1"], W["w2"], res["topk_w"], res["topk_ids"], topk_reduce=mode,
+                      stage_events=events if i >= 2 else [], **kw)
+        torch.cuda.synchronize()
+        acc = {}
+        for name, a, b in events:
+            acc.setdefault(name, []).append(a.elapsed_time(b))
+        acc = {k: sum(v) / len(v) for k, v in acc.items()}
+        r[mode] = round(acc["gemm2"] + acc.get("reduce", 0.0), 4)
+    return {"down_gemm_store_plus_reduce_ms": r["store"], "clear_plus_down_gemm_atomic_ms": r["atomic"]}
 
 
 def graph_replay_ms(torch, fused_moe, W, res, steps, block_m, method="auto"):
@@ -288,6 +310,10 @@ def main():
             dec4 = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, other)
             dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
             cpu = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds) if a.cpu_seconds > 0 else None
+            epi = None
+            if a.epilogue_comparison:
+                epi = {"tokens_%d" % a.tokens: epilogue_comparison(torch, fused_moe, W, main_res, 128),
+                       "tokens_%d" % a.decode_tokens: epilogue_comparison(torch, fused_moe, W, dec, 16)}
         del W
         torch.cuda.empty_cache()
 
@@ -347,6 +373,8 @@ def main():
                         "frac_of_hbm_peak": round(dw["bytes"] / (dec4["median_ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)},
         "configs": configs,
     }
+    if epi is not None:
+        out["down_epilogue_comparison"] = epi
     if cpu is not None:
         out["cpu_baseline"] = cpu
     print(json.dumps(out))

@@ -153,6 +153,18 @@ int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const ui
                           const uint32_t* schedule, void* out3_bf16, int tokens, int topk, int experts, int hidden,
                           int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
 
+/* Stage 2 with the top-k reduction in its epilogue: bf16(acc * routing weight) is added into out[tokens, hidden]
+ * (bf16, cleared by the caller) with packed bf16 atomics; no out3, no pyhip_moe_topk_reduce.  Replaces the atomic
+ * variant of the reference, src/contrib/moe_gemm_mxfp4.py:1334-1398 (and src/contrib/moe.py:703-787).  The result
+ * depends on the arrival order of a token's slots (each addition rounds to bf16); block_m is 16 or 128.  The
+ * deterministic out3 + reduce pair above is what pyhip_moe_forward uses. */
+int pyhip_moe_gemm2_mxfp4_atomic(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2,
+                                 const uint8_t* w2_scale, const void* bias2_bf16, const uint32_t* sorted_ids,
+                                 const float* sorted_weights, const uint32_t* sorted_expert_ids,
+                                 const uint32_t* num_valid_ids, const uint32_t* schedule, void* out_bf16, int tokens,
+                                 int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
+                                 pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * The same two GEMMs with bf16 activations ("w4a16"): weights are expanded from MXFP4 to bf16 in registers
  * and multiplied with the bf16 MFMA; nothing is quantised at run time.  Replaces moe_2stage_splitk with fp4

@@ -216,7 +216,10 @@ struct TileId
 // vector-memory counter ever covers the prefetches in flight.
 // NT: the weight loads are marked non-temporal (the launch decides: set when nearly every expert has a single row
 // block, so that no other workgroup reads the same weight tile)
-template <int STAGE, int MT, int ACT, bool NT>
+// ATOMIC (down GEMM only): the epilogue adds bf16(acc * routing weight) into out[token, :] with packed bf16 atomics
+// instead of storing it to out3[token, slot, :] for the top-k reduction: the reference's atomic variant
+// (src/contrib/moe_gemm_mxfp4.py:1334-1398).  The sum then depends on the order in which the slots arrive.
+template <int STAGE, int MT, int ACT, bool NT, bool ATOMIC = false>
 __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4_kernel(GemmArgs g)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
@@ -583,11 +586,22 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 transpose4x4_rows(lo);
                 transpose4x4_rows(hi);
                 // lane row q now holds channels q*16 + c*4 .. +3 in (lo[c], hi[c])
-                if(ok)
+                if(ok && !ATOMIC)
                 {
                     uint4* dst = (uint4*)(out + ((size_t)tok * g.topk + slot) * g.N + chw + kb * 16);
                     dst[0]     = make_uint4(lo[0], hi[0], lo[1], hi[1]);
                     dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
+                }
+                if(ok && ATOMIC)
+                {
+                    typedef short v2s __attribute__((ext_vector_type(2)));
+                    auto* dst = (__attribute__((address_space(1))) v2s*)(out + (size_t)tok * g.N + chw + kb * 16);
+#pragma unroll
+                    for(int c = 0; c < 4; c++)
+                    {
+                        __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c, __builtin_bit_cast(v2s, lo[c]));
+                        __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c + 1, __builtin_bit_cast(v2s, hi[c]));
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
             });
@@ -801,7 +815,7 @@ static int device_cu_count()
 }
 
 template <int STAGE>
-static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
+static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, bool atomic = false)
 {
     unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
     if(g.K < 1024 || g.E > SCHED_E_MAX)
@@ -839,6 +853,26 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream)
         else                                                     \
             GEMM_LAUNCH(MTV, 0, false);                          \
         break;
+    if constexpr(STAGE == 2)
+        if(atomic)
+        {
+            // the atomic epilogue exists for the two tile heights that matter for the comparison: decode and prefill
+            if(block_m == 16 && nt)
+                hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<2, 1, 0, true, true>), grid, block, 0, stream, g);
+            else if(block_m == 16)
+                hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<2, 1, 0, false, true>), grid, block, 0, stream, g);
+            else if(block_m == 128 && nt)
+                hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<2, 8, 0, true, true>), grid, block, 0, stream, g);
+            else if(block_m == 128)
+                hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<2, 8, 0, false, true>), grid, block, 0, stream, g);
+            else
+            {
+                pyhip_set_error("moe_gemm2 (atomic): block_m=%d not in {16,128}", block_m);
+                return PYHIP_ERR_INVALID;
+            }
+            PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel (atomic)");
+            return PYHIP_OK;
+        }
     switch(block_m)
     {
         GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(256, 16)
@@ -928,4 +962,38 @@ extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scal
     g.SC = (inter / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
     return launch_gemm<2>(g, block_m, 0, stream);
+}
+
+// The down GEMM with the top-k reduction in its epilogue: every (token, slot) result is added into out[token, :]
+// (bf16 [tokens, hidden], which the caller has cleared, e.g. with pyhip_moe_zero_fill) with packed bf16 atomics, the
+// reference's atomic variant (src/contrib/moe_gemm_mxfp4.py:1334-1398, src/contrib/moe.py:703-787).  No out3, no
+// reduction launch; the price is a result that depends on the arrival order of a token's slots (bf16 additions do
+// not commute with rounding) and atomic traffic.  block_m 16 or 128.
+extern "C" int pyhip_moe_gemm2_mxfp4_atomic(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2,
+                                            const uint8_t* w2_scale, const void* bias2_bf16, const uint32_t* sorted_ids,
+                                            const float* sorted_weights, const uint32_t* sorted_expert_ids,
+                                            const uint32_t* num_valid_ids, const uint32_t* schedule, void* out_bf16,
+                                            int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                            int64_t n_blk, hipStream_t stream)
+{
+    int rc = check_common("moe_gemm2_atomic", a2_q, a2_scale, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
+                          out_bf16, inter, block_m, n_blk, n_blk * block_m);
+    if(rc)
+        return rc;
+    PYHIP_REQUIRE(sorted_weights, "moe_gemm2_atomic: null sorted_weights");
+    PYHIP_REQUIRE(hidden > 0 && hidden % 256 == 0, "moe_gemm2_atomic: hidden=%d must be a multiple of 256", hidden);
+    PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0, "moe_gemm2_atomic: bad sizes");
+    if(n_blk == 0)
+        return PYHIP_OK;
+    GemmArgs g;
+    g.a_q = a2_q; g.a_s = a2_scale; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
+    g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
+    g.num_valid = num_valid_ids; g.out = out_bf16; g.out_q = nullptr; g.out_s = nullptr; g.OSK = 0;
+    g.limit = 0.f;
+    g.sched = schedule; g.E = experts;
+    g.T = tokens; g.topk = topk; g.K = inter; g.N = hidden;
+    g.SK = (inter + 511) / 512 * 16;
+    g.SC = (inter / 32 + 7) / 8 * 8;
+    g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
+    return launch_gemm<2>(g, block_m, 0, stream, true);
 }

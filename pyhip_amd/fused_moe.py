@@ -133,12 +133,15 @@ def fused_moe(
     return_parts=False,
     stage_events=None,
     swiglu_limit=None,
+    topk_reduce="store",
 ):
     """See the module docstring.  Extras beyond the reference signature: ``dtype=torch.float32`` returns
     the fp32 top-k sum without the final bf16 rounding; ``return_parts=True`` also returns the
     intermediate buffers; ``stage_events`` (a list) receives ``(name, start_event, end_event)`` per stage;
     ``activation=ActivationType.Swiglu`` selects gpt-oss's clamped SwiGLU with ``swiglu_limit`` (default 7.0, as
-    tests/contrib/moe/test_moe.py:76-81)."""
+    tests/contrib/moe/test_moe.py:76-81); ``topk_reduce="atomic"`` (MXFP4-activation path, row block 16 or 128,
+    bf16 output) lets the down GEMM add its results into the output with packed bf16 atomics, the reference's atomic
+    variant (src/contrib/moe_gemm_mxfp4.py:1334-1398), instead of the deterministic store + reduction."""
     lib = _lib.load()
     _require(activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts only")
     act = 1 if activation == ActivationType.Swiglu else 0
@@ -153,6 +156,7 @@ def fused_moe(
     out_dtype = hidden_states.dtype if dtype is None else dtype
     _require(out_dtype in (torch.bfloat16, torch.float32), "dtype must be bfloat16 or float32", TypeError)
     _require(method in ("auto", "a4w4", "w4a16", "jit", "gluon"), "method=%r" % (method,))
+    _require(topk_reduce in ("store", "atomic"), "topk_reduce=%r" % (topk_reduce,))
 
     # weights in the plain layout (no ``is_shuffled`` mark) are re-tiled once; the scales always come e8m0-shuffled,
     # as the reference passes them (tests/contrib/moe/test_moe.py:167-189)
@@ -210,7 +214,12 @@ def fused_moe(
         _require(num_local_tokens.is_cuda and num_local_tokens.dtype == torch.int32,
                  "num_local_tokens must be an int32 scalar tensor on the GPU", TypeError)
 
-    if not return_parts and stage_events is None:
+    atomic = topk_reduce == "atomic"
+    if atomic:
+        _require(not w4a16 and bm in (16, 128) and out_dtype == torch.bfloat16,
+                 "topk_reduce='atomic' needs the MXFP4-activation path, a row block of 16 or 128 and bf16 output")
+
+    if not return_parts and stage_events is None and not atomic:
         # the whole layer in one library call, intermediates in one workspace: two allocations and one foreign call
         # per layer instead of a dozen of each (the host side is what bounds small layers when they are not replayed
         # from a graph)
@@ -285,17 +294,28 @@ def fused_moe(
                                    _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, act, limit, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
-    out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
-    rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
-                                   _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
-                                   _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
-                                   T, k, global_E, H, I, bm, n_blk, stream)
-    _lib.check(rc, "moe_gemm2_mxfp4")
-    ev = _mark("gemm2", ev)
-    out = torch.empty(T, H, dtype=out_dtype, device=dev)
-    rc = _reduce(out3, out)
-    _lib.check(rc, "moe_topk_reduce")
-    _mark("reduce", ev)
+    if atomic:
+        out3 = None
+        out = torch.empty(T, H, dtype=out_dtype, device=dev)
+        _lib.check(lib.pyhip_moe_zero_fill(_lib.dptr(out), out.numel() * 2, stream), "moe_zero_fill")
+        rc = lib.pyhip_moe_gemm2_mxfp4_atomic(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                              _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                              _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out),
+                                              T, k, global_E, H, I, bm, n_blk, stream)
+        _lib.check(rc, "moe_gemm2_mxfp4_atomic")
+        _mark("gemm2", ev)
+    else:
+        out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
+        rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                       _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                       _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
+                                       T, k, global_E, H, I, bm, n_blk, stream)
+        _lib.check(rc, "moe_gemm2_mxfp4")
+        ev = _mark("gemm2", ev)
+        out = torch.empty(T, H, dtype=out_dtype, device=dev)
+        rc = _reduce(out3, out)
+        _lib.check(rc, "moe_topk_reduce")
+        _mark("reduce", ev)
     if narrow:
         out = out[:, : H - hidden_pad]
     if return_parts:

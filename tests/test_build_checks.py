@@ -12,7 +12,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SRC = os.path.join(ROOT, "pyhip_amd", "csrc", "moe_gemm_mxfp4.hip")
-KERNEL_RE = r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel"
+KERNEL_RE = r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]ELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel"
 
 
 @pytest.fixture(scope="module")
@@ -27,7 +27,8 @@ def gemm_asm(tmp_path_factory):
     assert r.returncode == 0, r.stdout[-2000:]
     text = out.read_text()
     kernels = re.findall(KERNEL_RE, text, re.S | re.M)
-    assert len(kernels) == 30, "expected (gate_up x two activations + down) x five tile heights x two load policies"
+    assert len(kernels) == 34, ("expected (gate_up x two activations + down) x five tile heights x two load policies, "
+                                "plus the down GEMM with the atomic epilogue at two tile heights x two load policies")
     return text, kernels
 
 

@@ -545,3 +545,26 @@ def test_odd_views_of_hidden_states_are_copied():
         b = fused_moe(view.contiguous(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, method=method)
         torch.cuda.synchronize()
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("name,T,bm", [("dsv3_s", 16, 16), ("tiny", 300, 128), ("odd", 200, 128)])
+def test_atomic_topk_reduce_variant(name, T, bm):
+    """topk_reduce="atomic": the down GEMM adds bf16(acc * routing weight) into the output with packed bf16 atomics
+    (the reference's atomic variant, src/contrib/moe_gemm_mxfp4.py:1334-1398).  Every addition rounds to bf16 and the
+    slots arrive in no fixed order, so the comparison with the deterministic result allows one bf16 rounding (half an
+    ulp, 2^-8 relative) of a running sum no larger than the sum of the slot magnitudes per addition."""
+    L = cases.make_layer(name, T, seed=17)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    print(f"atomic-reduce case {name} T={T} bm={bm}", flush=True)
+    kw = dict(w1_scale=w1s, w2_scale=w2s, block_size_M=bm, method="a4w4")
+    ref32, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, dtype=torch.float32, return_parts=True, **kw)
+    got = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, topk_reduce="atomic", **kw)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and torch.isfinite(got.float()).all()
+    mag = parts["out3"].float().abs().sum(dim=1)                      # sum over slots of |slot value|
+    assert ((got.float() - ref32).abs() <= mag * L.k * 2.0 ** -8 + 1e-30).all()
+    rms = ref32.pow(2).mean().sqrt().item()
+    err = (got.float() - ref32).abs().max().item() / rms
+    print(f"  max|atomic - deterministic fp32 sum| / rms = {err:.3e}", flush=True)
+    assert metrics.cosine(_f(got), _f(ref32)) >= 0.9999
