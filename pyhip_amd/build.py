@@ -28,6 +28,31 @@ def _run(cmd):
     return out
 
 
+CO_DIR = os.path.join(HERE, "co")
+# sources whose kernels are also shipped as stand-alone code objects (see build_co)
+CO_SOURCES = ["moe_quant.hip", "moe_reduce.hip", "moe_gemm_mxfp4.hip"]
+
+
+def build_co(verbose=False, jobs=4):
+    """Device-only code objects ``pyhip_amd/co/*.co`` for gfx950: what ``hipModuleLoad`` takes, for callers that launch
+    kernels themselves with ``hipModuleLaunchKernel`` and a packed argument struct (``pyhip_amd/co_module.py``; the
+    reference's loader works that way, src/core/hiptools.py:54-100)."""
+    os.makedirs(CO_DIR, exist_ok=True)
+    flags = [f for f in FLAGS if f != "-fPIC"]
+
+    def one(src):
+        out = os.path.join(CO_DIR, src.replace(".hip", ".co"))
+        return _run([HIPCC, *flags, "--offload-device-only", "--no-gpu-bundle-output", "-c", os.path.join(CSRC, src), "-o", out])
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        outs = list(ex.map(one, CO_SOURCES))
+    if verbose:
+        for o in outs:
+            if o.strip():
+                print(o)
+    return CO_DIR
+
+
 def build(verbose=False, jobs=4):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -49,3 +74,4 @@ def build(verbose=False, jobs=4):
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_co(verbose=True))

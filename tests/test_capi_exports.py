@@ -64,3 +64,19 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libpyhip_moe.so")
     with pytest.raises(_lib.PyhipError, match="no fallback"):
         _lib.load()
+
+
+def test_code_objects_hold_the_kernels():
+    """pyhip_amd/co/*.co (built next to the library) are loadable gfx950 code objects that export the kernels under the
+    names pyhip_amd/co_module.py computes"""
+    from pyhip_amd import co_module as co
+    for name, wanted in (("moe_quant", [b"moe_act_quant_mxfp4_kernel"]),
+                         ("moe_reduce", [co.reduce_kernel_name(f, r).encode() for f in (0, 1) for r in (0, 1)]),
+                         ("moe_gemm_mxfp4", [co.gemm_kernel_name(s, mt).encode() for s in (1, 2) for mt in (1, 2, 4, 8, 16)]
+                          + [co.gemm_kernel_name(2, 8, 0, False, True).encode()])):
+        path = os.path.join(co.CO_DIR, name + ".co")
+        assert os.path.exists(path), path + " missing: run python -m pyhip_amd.build"
+        blob = open(path, "rb").read()
+        assert blob[:4] == b"\x7fELF" and b"gfx950" in blob
+        for w in wanted:
+            assert w + b"\x00" in blob, w
