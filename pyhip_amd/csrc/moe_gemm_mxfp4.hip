@@ -588,6 +588,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 // lane row q now holds channels q*16 + c*4 .. +3 in (lo[c], hi[c])
                 if(ok && !ATOMIC)
                 {
+                    // (plain stores: marked non-temporal they cost the down GEMM 5 % and the reduction, which then finds
+                    // nothing of out3 in the last-level cache, another 4 %)
                     uint4* dst = (uint4*)(out + ((size_t)tok * g.topk + slot) * g.N + chw + kb * 16);
                     dst[0]     = make_uint4(lo[0], hi[0], lo[1], hi[1]);
                     dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
