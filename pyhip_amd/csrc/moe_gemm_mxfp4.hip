@@ -45,35 +45,15 @@ struct GemmArgs
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
 };
 
-// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales; OPW / OPA select
-// the byte of the scale dwords.  Written in assembly with the accumulator tied to the destination: left to
-// the compiler, about a third of the accumulators get renamed on every K-step and the kernel no longer fits
-// its register budget.
-template <int OPW, int OPA>
-__device__ __forceinline__ void mfma_fp4(v4f& acc, v4i w, v4i a, int w_scale, int a_scale)
-{
-    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4 blgp:4"
-                 : "+v"(acc)
-                 : "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1), "n"(OPW >> 1), "n"(OPA >> 1));
-}
-
-// The same with the accumulator in the accumulation registers a[ACC0 .. ACC0+3], named in the instruction text:
-// the compiler never sees these registers as values.  Tiles of 256 rows need 256 accumulator registers per lane
-// on top of the operand registers; declared as ordinary vectors (in either register file) the compiler keeps
-// shuffling them between the files around the loop and spills.  With the register numbers fixed by hand, the
-// kernel reserves all 256 accumulation registers once (see the clobber at its top) and must keep its ordinary
-// register use below the point where the compiler would start parking values in them (checked at build time by
-// looking for accumulation-register moves outside these helpers).
-template <int OPW, int OPA, int ACC0>
-__device__ __forceinline__ void mfma_fp4_fixed(v4i w, v4i a, int w_scale, int a_scale)
-{
-    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%0:%1], %2, %3, a[%0:%1], %4, %5 op_sel:[%6,%7,0] op_sel_hi:[%8,%9,0] cbsz:4 blgp:4"
-                 :
-                 : "n"(ACC0), "n"(ACC0 + 3), "v"(w), "v"(a), "v"(w_scale), "v"(a_scale), "n"(OPW & 1), "n"(OPA & 1),
-                   "n"(OPW >> 1), "n"(OPA >> 1));
-}
-// The four MFMAs of one activation row group (16 rows) against the wave's four weight row groups, one assembly
-// statement.  accumulator of (weight row group j, row group mt): a[(j*MT + mt)*4 .. +3]; scale bytes: see mfma_fp4.
+// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales, four at a time: the
+// four MFMAs of one activation row group (16 rows) against the wave's four weight row groups, one assembly statement.
+// The accumulators are the accumulation registers a[(j*MT + mt)*4 .. +3] of (weight row group j, row group mt), named
+// in the instruction text: the compiler never sees them as values.  (Declared as ordinary vectors, in either register
+// file, about a third of them get renamed on every K-step, get shuffled between the files around the loop and spill.)
+// With the register numbers fixed by hand, the kernel reserves the range once (see the clobber at its top) and must keep
+// its ordinary register use below the point where the compiler would start parking values there (checked at build time
+// by looking for accumulation-register moves outside these helpers).  U = K-step inside the K-group: it selects the byte
+// of the scale dwords (weights: (kt%2)*2 + (row%32)/16 through op_sel / op_sel_hi, activations: kt%4).
 // (Row groups that hold only padding are NOT skipped.  Measured with a compare and a branch around the four MFMAs
 // inside this statement, so that nothing else about the generated code changes: the pair costs more issue time in
 // full tiles than the skipped MFMAs save elsewhere: DeepSeek-V3 shape, 8192 tokens, where a fifth of the row groups
@@ -225,9 +205,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass only needs the launch stub
     constexpr int BM    = MT * 16;
     // The accumulators live in the accumulation registers a0 .. a[16*MT-1], named by hand in the instruction text
-    // (mfma_fp4_fixed); the clobber reserves that range for the kernel.  RING: the one-wave-per-SIMD 256-row tile
-    // reads its LDS operands through a deeper ring of registers.
-    constexpr bool RING = true;
+    // (mfma_row_group); the clobber reserves that range for the kernel.
     if constexpr(MT == 16) asm volatile("" ::: "a0", "a255");
     if constexpr(MT == 8) asm volatile("" ::: "a0", "a127");
     if constexpr(MT == 4) asm volatile("" ::: "a0", "a63");
@@ -686,17 +664,20 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         // MFMAs, prefetches and weight loads of the K-group
         constexpr int MA  = MT;                   // row groups that take part
         constexpr int PPM = (NPF + MA - 1) / MA;  // prefetch operations issued after each row group's MFMAs
+        // The activation operand of a row group and its scale dword (one per 16-row group and K-group, op_sel picks the
+        // K-step's byte) are read RA row groups ahead of the MFMAs that consume them, across K-step boundaries, through
+        // a ring of RA + 1 register sets: two ahead with two waves per SIMD, four in the one-wave-per-SIMD 256-row
+        // tile, where nothing else covers the LDS latency.
         constexpr int RA = MT > 8 ? 4 : 2;
         v4i af_r[RA + 1];
-        int asc_all[RING ? MT : 1];              // the scale dword of a row group serves all four K-steps
+        int asc_all[MT];                          // the scale dword of a row group serves all four K-steps
         auto lds_read = [&](auto NN) __attribute__((always_inline)) {
             constexpr int n = decltype(NN)::value, uu = n / MA, mm = n % MA;
             af_r[n % (RA + 1)] = *(const v4i*)(stage[p] + (uu * SLOTS + mm) * 1024 + rd_a);
             if constexpr(uu == 0)
-                asc_all[RING ? mm : 0] = *(const int*)(sstage[p] + mm * 256 + rd_s);
+                asc_all[mm] = *(const int*)(sstage[p] + mm * 256 + rd_s);
         };
-        if constexpr(RING)
-            static_for<RA>([&](auto NN) __attribute__((always_inline)) { lds_read(NN); });
+        static_for<RA>([&](auto NN) __attribute__((always_inline)) { lds_read(NN); });
         __builtin_amdgcn_sched_barrier(0);
         static_for<4>([&](auto U) __attribute__((always_inline)) {
             constexpr int u = decltype(U)::value;
@@ -711,34 +692,13 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             wait_vm_tiles<YOUNGER>(wf[u][0], wf[u][1], wf[u][2], wf[u][3]);
             if(u == 0)
                 wait_vm_scales<YOUNGER>(w_sc[p][0], w_sc[p][1], w_sc[p][2], w_sc[p][3]);
-            // activation operand and its scale dword (one per 16-row group and K-group, op_sel picks this K-step's
-            // byte) are read ahead of the MFMAs that consume them: one row group ahead within a K-step with two
-            // waves per SIMD, RA row groups ahead across K-step boundaries (a ring of RA + 1 register sets) in
-            // the one-wave-per-SIMD 256-row tile, where nothing else covers the LDS latency
-            v4i af  = {0, 0, 0, 0};
-            int asc = 0;
-            if constexpr(!RING)
-            {
-                af  = *(const v4i*)(stage[p] + (u * SLOTS) * 1024 + rd_a);
-                asc = *(const int*)(sstage[p] + rd_s);
-            }
             static_for<MA>([&](auto M) __attribute__((always_inline)) {
                 constexpr int mt = decltype(M)::value;
-                v4i af_n  = af;
-                int asc_n = asc;
-                if constexpr(RING)
-                {
-                    constexpr int n = u * MA + mt;             // position in the K-group's sequence of row groups
-                    if constexpr(n + RA < 4 * MA)
-                        lds_read(std::integral_constant<int, n + RA>{});
-                    af  = af_r[n % (RA + 1)];
-                    asc = asc_all[RING ? mt : 0];
-                }
-                else if constexpr(mt + 1 < MA)
-                {
-                    af_n  = *(const v4i*)(stage[p] + (u * SLOTS + mt + 1) * 1024 + rd_a);
-                    asc_n = *(const int*)(sstage[p] + (mt + 1) * 256 + rd_s);
-                }
+                constexpr int n  = u * MA + mt;                // position in the K-group's sequence of row groups
+                if constexpr(n + RA < 4 * MA)
+                    lds_read(std::integral_constant<int, n + RA>{});
+                const v4i af  = af_r[n % (RA + 1)];
+                const int asc = asc_all[mt];
                 __builtin_amdgcn_sched_barrier(0);
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
                 mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
@@ -758,11 +718,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                             load_wtile(std::integral_constant<int, u - 1>{}, J, kpre * 4 + u - 1);
                     });
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr(!RING)
-                {
-                    af  = af_n;
-                    asc = asc_n;
-                }
             });
             __builtin_amdgcn_sched_barrier(0);
             if constexpr(u == 3)
