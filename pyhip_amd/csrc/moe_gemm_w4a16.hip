@@ -4,11 +4,14 @@
 // (src/contrib/moe.py:362-787, moe_2stage_splitk with fp4 weights, driven by
 // tests/contrib/moe/test_moe.py:347-374); at such sizes the layer only streams weights, so the kernel is kept
 // simple: one workgroup per (row block, weight tile), the K loop software-pipelined one K-step ahead.
-// Two mappings of a workgroup's four waves:
-//   SPLITK = false: tile of 256 weight rows, wave w owns 64 of them over the whole K range;
-//   SPLITK = true : tile of 64 weight rows shared by all waves, wave w takes K-steps w, w+4, ... and the four
-//                   partial sums meet in LDS (the reference's split-K arrangement, src/contrib/moe.py:362-500).
-//                   Four times as many workgroups: used when the layer would otherwise not fill the GPU.
+// Three mappings of a workgroup's waves:
+//   SPLIT = 0 : four waves, tile of 256 weight rows, wave w owns 64 of them over the whole K range;
+//   SPLIT = 4 : four waves share a tile of 64 weight rows, wave w takes K-steps w, w+4, ... and the four
+//               partial sums meet in LDS (the reference's split-K arrangement, src/contrib/moe.py:362-500).
+//               Four times as many workgroups: used when the layer would otherwise not fill the GPU.
+//   SPLIT = 16: the same with sixteen waves per workgroup, for a long K with so few tiles that even the four-way
+//               split leaves most CUs without a wave (Mixtral's down GEMM at one token: 128 tiles of 112 K-steps;
+//               every wave is a chain of dependent K-steps, and the chain, not the bandwidth, sets the time).
 //
 // Operand mapping.  A pre-shuffled 1 KB weight block (src/misc.py:116-130) gives lane (row = l % 16,
 // kb = l / 16) the 32 consecutive K-elements kb*32 .. kb*32+31 of its row.  The bf16 MFMA 16x16x32 wants 8
@@ -52,11 +55,12 @@ __device__ __forceinline__ void expand_fp4(const v4i& w, u32 scale_byte, v8bf (&
 }
 
 // STAGE 1 = gate_up (+ SiLU(gate) * up), 2 = down (* routing weight).  MT = row groups of 16 per tile.
-template <int STAGE, int MT, bool SPLITK>
-__global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
+template <int STAGE, int MT, int SPLIT>
+__global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
 {
-    constexpr int BM = MT * 16;
-    __shared__ float red[SPLITK ? 4 * 4 * MT * WAVE * 4 : 1];      // [wave][j][mt][lane][4]
+    constexpr int BM      = MT * 16;
+    constexpr bool SPLITK = SPLIT != 0;
+    __shared__ float red[SPLITK ? SPLIT * 4 * MT * WAVE * 4 : 1];  // [wave][j][mt][lane][4]
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int r = lane & 15, kb = lane >> 4;
@@ -109,7 +113,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
             acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int KT = g.K / 128;
-    constexpr int KSTRIDE = SPLITK ? 4 : 1;
+    constexpr int KSTRIDE = SPLITK ? SPLIT : 1;
     v4i wf[2][4];
     v4i af[2][MT][4];
     u32 wsc[2][4];             // scale dwords (one covers the two K-steps of a 256-K column tile), loaded with
@@ -166,7 +170,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
             for(int mt = 0; mt < MT; mt++)
                 *(v4f*)&red[(((wave * 4 + j) * MT + mt) * WAVE + lane) * 4] = acc[j][mt];
         __syncthreads();
-        if(STAGE == 1 && wave >= 2)
+        if(wave >= (STAGE == 1 ? 2 : 4))
             return;
 #pragma unroll
         for(int j = 0; j < 4; j++)
@@ -175,7 +179,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
             {
                 v4f sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for(int w = 0; w < 4; w++)
+                for(int w = 0; w < SPLIT; w++)
                     sum += *(const v4f*)&red[(((w * 4 + j) * MT + mt) * WAVE + lane) * 4];
                 acc[j][mt] = sum;
             }
@@ -236,7 +240,7 @@ __global__ void __launch_bounds__(W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args
     }
 }
 
-// split_k: 0 = decide here, 1 = never, 4 = always
+// split_k: 0 = decide here, 1 = never, 4 / 16 = always that many waves per 64-row tile
 template <int STAGE>
 static int launch_w4a16(W4A16Args g, int block_m, int64_t n_blk, int64_t rows, int experts, int split_k,
                         hipStream_t stream)
@@ -245,21 +249,33 @@ static int launch_w4a16(W4A16Args g, int block_m, int64_t n_blk, int64_t rows, i
     int64_t blocks = rows < n_blk ? rows : n_blk;
     if(experts + rows / block_m < blocks)
         blocks = experts + rows / block_m;
-    const bool split = split_k == 4 || (split_k == 0 && blocks * g.n_tiles < 2048);
+    int split = split_k == 1 ? 0 : split_k;
+    if(split_k == 0 && blocks * g.n_tiles < 2048)
+        // sixteen waves when the four-way split would still start fewer workgroups than there are CUs and the K loop
+        // is long enough to matter (Mixtral shape, one token: the layer 54.0 -> 49.7 us; forced onto the gate_up GEMM as well,
+        // which already starts 896 workgroups there, 57.5 us)
+        split = (blocks * g.n_tiles * 4 < 256 && g.K >= 8192 && block_m == 16) ? 16 : 4;
+    // (sixteen waves of a workgroup share the register file four to a SIMD: 128 registers each, which only the 16-row
+    // tile fits into; and every wave needs a K-step of its own)
+    if(split == 16 && (g.K < 2048 || block_m != 16))
+    {
+        pyhip_set_error("moe_gemm_w4a16: split_k=16 needs K >= 2048 and block_m = 16 (K=%d, block_m=%d)", g.K, block_m);
+        return PYHIP_ERR_INVALID;
+    }
     if(split)
         g.n_tiles *= 4;
     // blocks past the bound cannot hold rows (the sort fills blocks from 0 upwards): no workgroups for them
-    dim3 grid((unsigned)(blocks * g.n_tiles)), block(W4A16_THREADS);
-    switch(block_m * 2 + (split ? 1 : 0))
+    dim3 grid((unsigned)(blocks * g.n_tiles)), block(split == 16 ? 1024 : W4A16_THREADS);
+#define W4A16_CASE(BMV, MTV, SPV) \
+    case BMV * 32 + SPV: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, MTV, SPV>), grid, block, 0, stream, g); break;
+    switch(block_m * 32 + split)
     {
-    case 32: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1, false>), grid, block, 0, stream, g); break;
-    case 33: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 1, true>), grid, block, 0, stream, g); break;
-    case 64: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2, false>), grid, block, 0, stream, g); break;
-    case 65: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 2, true>), grid, block, 0, stream, g); break;
-    case 128: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4, false>), grid, block, 0, stream, g); break;
-    case 129: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, 4, true>), grid, block, 0, stream, g); break;
+        W4A16_CASE(16, 1, 0) W4A16_CASE(16, 1, 4) W4A16_CASE(16, 1, 16)
+        W4A16_CASE(32, 2, 0) W4A16_CASE(32, 2, 4)
+        W4A16_CASE(64, 4, 0) W4A16_CASE(64, 4, 4)
     default: pyhip_set_error("moe_gemm_w4a16: block_m=%d not in {16,32,64}", block_m); return PYHIP_ERR_INVALID;
     }
+#undef W4A16_CASE
     PYHIP_CHECK_LAUNCH("moe_gemm_w4a16_kernel");
     return PYHIP_OK;
 }
@@ -285,7 +301,7 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
                                      int64_t n_blk, int split_k, int activation, float swiglu_limit,
                                      hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4, "moe_gemm1_w4a16: split_k=%d not in {0,1,4}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm1_w4a16: split_k=%d not in {0,1,4,16}", split_k);
     PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
                   "moe_gemm1_w4a16: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
     int rc = check_w4a16("moe_gemm1_w4a16", hidden_bf16, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
@@ -311,7 +327,7 @@ extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, con
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
                                      int64_t n_blk, int split_k, hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4, "moe_gemm2_w4a16: split_k=%d not in {0,1,4}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm2_w4a16: split_k=%d not in {0,1,4,16}", split_k);
     int rc = check_w4a16("moe_gemm2_w4a16", a2_bf16, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                          out3_bf16, inter, block_m, n_blk, hidden / 256);
     if(rc)

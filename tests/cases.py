@@ -18,6 +18,9 @@ CONFIGS = {
     # an expert count that is not a multiple of the 8 XCDs the tile schedule deals experts to, an odd top-k,
     # three K-groups in the gate_up GEMM
     "odd": dict(E=12, k=3, H=1536, I=1024, router="softmax"),
+    # long K in both GEMMs (16 and 20 K-steps of 128): the sixteen-wave split of the bf16-activation kernels, with one
+    # K-step per wave in gate_up and an uneven share (one or two) in down
+    "longk_s": dict(E=4, k=2, H=2048, I=2560, router="softmax"),
 }
 
 

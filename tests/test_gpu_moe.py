@@ -222,6 +222,7 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     ("tiny", 64, 16, True, 4), ("tiny", 200, 64, False, 4), ("mixtral_s", 33, 32, False, 4), ("dsv3_s", 16, None, False, 4),
     ("gptoss_s1", 20, 16, True, 4),
     ("odd", 9, 16, False, 0), ("odd", 77, 32, True, 1),
+    ("longk_s", 3, 16, True, 16), ("longk_s", 40, 16, False, 16), ("longk_s", 3, 16, False, 4),
 ])
 def test_w4a16_matches_oracle(name, T, bm, bias, splitk):
     """bf16 activations x MXFP4 weights (method="w4a16") against the oracle's "a16" path:
