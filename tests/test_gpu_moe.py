@@ -602,3 +602,38 @@ def test_reference_style_inputs(T):
               f"cosine={metrics.cosine(got, ref):.8f} calc_diff={cd:.2e}", flush=True)
         assert np.isfinite(got).all() and cd <= 0.01 and metrics.cosine(got, ref) >= TOL_COS
         assert np.mean(err > TOL_MAX) <= 2e-3 and err.max() <= 0.1
+
+
+@pytest.mark.parametrize("T,bm", [(48, 16), (300, 128)])
+def test_more_experts_than_the_tile_schedule_holds(T, bm):
+    """720 experts: the MXFP4 GEMMs keep their tile schedule in LDS for up to 704 and otherwise start one workgroup
+    per tile.  (The 720 experts are 45 copies of 16 drawn ones, so that building the case stays cheap; every token's
+    experts are distinct.)  Same bounds as the other end-to-end cases; and the result must equal, bit for bit, the
+    one the 16-expert layer gives for the ids folded back, which takes the scheduled path."""
+    base = cases.make_layer("tiny", T, seed=11, E=16, k=4, bias=True)
+    rep = 45
+    L = cases.Layer()
+    L.E, L.k, L.H, L.I, L.T = base.E * rep, base.k, base.H, base.I, T
+    L.hidden, L.topk_w = base.hidden, base.topk_w
+    L.w1q, L.w1s = np.tile(base.w1q, (rep, 1, 1)), np.tile(base.w1s, (rep, 1, 1))
+    L.w2q, L.w2s = np.tile(base.w2q, (rep, 1, 1)), np.tile(base.w2s, (rep, 1, 1))
+    L.bias1, L.bias2 = base.bias1.repeat(rep, 1), base.bias2.repeat(rep, 1)
+    rng = np.random.default_rng(5)
+    L.topk_ids = (base.topk_ids + base.E * rng.integers(0, rep, size=base.topk_ids.shape)).astype(base.topk_ids.dtype)
+    assert L.topk_ids.max() >= 704
+    outs = []
+    for lay in (L, base):
+        w1, w1s, w2, w2s = cases.device_weights(lay)
+        tw, ti = torch.from_numpy(lay.topk_w).cuda(), torch.from_numpy(lay.topk_ids).cuda()
+        print(f"many-experts case E={lay.E} T={T} bm={bm}", flush=True)
+        outs.append(fused_moe(lay.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, block_size_M=bm,
+                              bias1=lay.bias1.cuda(), bias2=lay.bias2.cuda(), dtype=torch.float32, method="a4w4",
+                              return_parts=True))
+        torch.cuda.synchronize()
+    (out32, parts), (out_base, _) = outs
+    assert torch.equal(out32, out_base)
+    w1e, w2e, ref_a2, nflip1 = _stage_checks(L, parts, parts["block_m"])
+    assert w1e <= TOL_MAX and w2e <= TOL_MAX
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4", bias1=_f(L.bias1),
+                      bias2=_f(L.bias2))
+    _end_to_end(_f(out32), ref, ref_a2, nflip1)
