@@ -59,6 +59,9 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="target size of the CPU sample; 0 = skip")
     ap.add_argument("--epilogue-comparison", action="store_true",
                     help="also time the down GEMM with the atomic top-k epilogue against store + reduction")
+    ap.add_argument("--tile256-comparison", type=int, default=0, metavar="TOKENS",
+                    help="also time the GEMMs of the headline shape at TOKENS tokens on the 128-row tile, the four-wave "
+                         "256-row tile and the eight-wave 256-row tile with both operands through LDS")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
     return ap.parse_args()
@@ -180,6 +183,32 @@ def epilogue_comparison(torch, fused_moe, W, res, block_m):
         acc = {k: sum(v) / len(v) for k, v in acc.items()}
         r[mode] = round(acc["gemm2"] + acc.get("reduce", 0.0), 4)
     return {"down_gemm_store_plus_reduce_ms": r["store"], "clear_plus_down_gemm_atomic_ms": r["atomic"]}
+
+
+def tile256_comparison(torch, fused_moe, W, shape, tokens):
+    """gate_up + down GEMM time of the same layer on three tiles (events around the launches of the step-by-step path,
+    untimed passes): 128 rows (weights into registers, two workgroups per CU), 256 rows with four waves (weights into
+    registers, one wave per SIMD), 256 rows with eight waves and both operands staged through LDS"""
+    from pyhip_amd import workloads
+    hidden, tw, ti = workloads.make_inputs(shape, tokens)
+    if W["hidden_pad"]:
+        hidden = torch.nn.functional.pad(hidden, (0, W["hidden_pad"]))
+    out, ref = {}, None
+    for name, kw in (("rows128_registers", dict(block_size_M=128)), ("rows256_registers_4waves", dict(block_size_M=256)),
+                     ("rows256_lds_8waves", dict(operand_staging="lds"))):
+        base = call_kwargs(W, 0, "a4w4")
+        base.update(kw)
+        events = []
+        for i in range(10):
+            o = fused_moe(hidden, W["w1"], W["w2"], tw, ti, stage_events=events if i >= 2 else [], **base)
+        torch.cuda.synchronize()
+        ref = o if ref is None else ref
+        assert torch.equal(o, ref), "tiles disagree"
+        acc = {}
+        for nm, a, b in events:
+            acc.setdefault(nm, []).append(a.elapsed_time(b))
+        out[name] = {k: round(sum(v) / len(v), 4) for k, v in acc.items() if k in ("gemm1", "gemm2")}
+    return out
 
 
 def graph_replay_ms(torch, fused_moe, W, res, steps, block_m, method="auto"):
@@ -320,6 +349,7 @@ def main():
             dec4 = time_point(torch, fused_moe, W, a.shape, a.decode_tokens, max(a.steps, 50), max(a.warmup, 10), a.block_m, other)
             dec_graph_ms = graph_replay_ms(torch, fused_moe, W, dec, max(a.steps, 50), a.block_m)
             cpu = cpu_baseline(torch, W, a.shape, main_res, a.cpu_seconds) if a.cpu_seconds > 0 else None
+            tile256 = tile256_comparison(torch, fused_moe, W, a.shape, a.tile256_comparison) if a.tile256_comparison else None
             epi = None
             if a.epilogue_comparison:
                 epi = {"tokens_%d" % a.tokens: epilogue_comparison(torch, fused_moe, W, main_res, 128),
@@ -385,6 +415,8 @@ def main():
     }
     if epi is not None:
         out["down_epilogue_comparison"] = epi
+    if tile256:
+        out["tile256_comparison_ms"] = {"tokens": a.tile256_comparison, **tile256}
     if cpu is not None:
         out["cpu_baseline"] = cpu
     print(json.dumps(out))

@@ -153,6 +153,24 @@ int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const ui
                           const uint32_t* schedule, void* out3_bf16, int tokens, int topk, int experts, int hidden,
                           int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
 
+/* The same two GEMMs on the eight-wave tile of 256 rows x 256 weight rows whose operands BOTH go through LDS (LDS-DMA
+ * into a ring of five weight stages and three activation stages, two wave rows half a K-step apart), the tile shape of
+ * the reference's prefill kernel (src/contrib/moe_gemm_mxfp4.py:318-637).  Arguments as pyhip_moe_gemm1_mxfp4 /
+ * pyhip_moe_gemm2_mxfp4 with block_m = 256: the sort must have been run with block_size 256 and must have written the
+ * schedule (required here); hidden / inter (the K of the GEMM) >= 1024; at most 512 experts.  Results are bit-identical
+ * to the other tiles'.  Measured slower than the four-wave 256-row tile (DeepSeek-V3 shape, 6144 tokens: layer 1.86
+ * against 1.70 ms), so no other entry point selects it. */
+int pyhip_moe_gemm1_mxfp4_lds(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
+                              const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
+                              const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q,
+                              uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter,
+                              int64_t n_blk, int activation, float swiglu_limit, pyhip_stream_t stream);
+int pyhip_moe_gemm2_mxfp4_lds(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                              const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
+                              const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
+                              const uint32_t* schedule, void* out3_bf16, int tokens, int topk, int experts,
+                              int hidden, int inter, int64_t n_blk, pyhip_stream_t stream);
+
 /* Stage 2 with the top-k reduction in its epilogue: bf16(acc * routing weight) is added into out[tokens, hidden]
  * (bf16, cleared by the caller) with packed bf16 atomics; no out3, no pyhip_moe_topk_reduce.  Replaces the atomic
  * variant of the reference, src/contrib/moe_gemm_mxfp4.py:1334-1398 (and src/contrib/moe.py:703-787).  The result

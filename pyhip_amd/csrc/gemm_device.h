@@ -1,0 +1,188 @@
+// Device-side building blocks shared by the MXFP4 x MXFP4 GEMM kernels (moe_gemm_mxfp4.hip, moe_gemm_mxfp4_wide.hip):
+// the kernel argument block, the scaled MFMA on hand-numbered accumulation registers, the vector-memory primitives
+// whose waits are counted by hand, and the lane transposes of the epilogues.
+#pragma once
+#include "common.h"
+#include <stdlib.h>
+
+#define GEMM_THREADS 256
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+struct GemmArgs
+{
+    const uint8_t* a_q;        // activations, e2m1 pairs  [a_rows, K/2]
+    const uint8_t* a_s;        // activation scales        [a_rows, SK]  (layout: moe_quant.hip)
+    const uint8_t* w;          // weights, pre-shuffled    [E, N, K/2]
+    const uint8_t* w_s;        // weight scales, shuffled  [E*N (padded to 256), SC]
+    const uint16_t* bias;      // bf16 [E, N] or null
+    const u32* sorted_ids;     // [n_blk * BM]
+    const float* sorted_w;     // [n_blk * BM]
+    const u32* sorted_e;       // [n_blk]
+    const u32* num_valid;      // [2]
+    const u32* sched;          // tile schedule written by the sort (moe_sort.hip: write_schedule) or null
+    void* out;                 // stage 1: bf16 [n_blk*BM, N/2] (may be null); stage 2: bf16 [T, topk, N]
+    uint8_t* out_q;            // stage 1: MXFP4 of the output, e2m1 pairs [n_blk*BM, N/4], or null
+    uint8_t* out_s;            //          and its scales [n_blk*BM, OSK] in the activation-scale layout
+    int OSK;
+    float limit;               // stage 1, SwiGLU: the clamp
+    int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
+};
+
+// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales, four at a time: the
+// four MFMAs of one activation row group (16 rows) against the wave's four weight row groups, one assembly statement.
+// The accumulators are the accumulation registers a[(j*MT + mt)*4 .. +3] of (weight row group j, row group mt), named
+// in the instruction text: the compiler never sees them as values.  (Declared as ordinary vectors, in either register
+// file, about a third of them get renamed on every K-step, get shuffled between the files around the loop and spill.)
+// With the register numbers fixed by hand, the kernel reserves the range once (see the clobber at its top) and must keep
+// its ordinary register use below the point where the compiler would start parking values there (checked at build time
+// by looking for accumulation-register moves outside these helpers).  U = K-step inside the K-group: it selects the byte
+// of the scale dwords (weights: (kt%2)*2 + (row%32)/16 through op_sel / op_sel_hi, activations: kt%4).
+// (Row groups that hold only padding are NOT skipped.  Measured with a compare and a branch around the four MFMAs
+// inside this statement, so that nothing else about the generated code changes: the pair costs more issue time in
+// full tiles than the skipped MFMAs save elsewhere: DeepSeek-V3 shape, 8192 tokens, where a fifth of the row groups
+// are padding: gate_up 1.30 -> 1.38 ms; Mixtral shape, 4096 tokens, no padding: 0.477 -> 0.503 ms.)
+template <int U, int MTI, int MT>
+__device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale)
+{
+    constexpr int A0 = (0 * MT + MTI) * 4, A1 = (1 * MT + MTI) * 4, A2 = (2 * MT + MTI) * 4, A3 = (3 * MT + MTI) * 4;
+    constexpr int W0 = (U & 1) * 2 + 0, W1 = (U & 1) * 2 + 1;       // weight-scale byte: (kt%2)*2 + (row%32)/16
+#define MFMA_TEXT(ACC, ACCE, W, WS, WL, WH)                                                                            \
+    "v_mfma_scale_f32_16x16x128_f8f6f4 a[%[" #ACC "]:%[" #ACCE "]], %[" #W "], %[a], a[%[" #ACC "]:%[" #ACCE "]], %[" #WS  \
+    "], %[as] op_sel:[%[" #WL "],%[al],0] op_sel_hi:[%[" #WH "],%[ah],0] cbsz:4 blgp:4\n\t"
+    asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
+                 MFMA_TEXT(c2, e2, w2, s23, x0l, x0h) MFMA_TEXT(c3, e3, w3, s23, x1l, x1h)
+                 :
+                 : [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3), [c2] "n"(A2), [e2] "n"(A2 + 3),
+                   [c3] "n"(A3), [e3] "n"(A3 + 3), [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
+                   [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [x0l] "n"(W0 & 1), [x0h] "n"(W0 >> 1),
+                   [x1l] "n"(W1 & 1), [x1h] "n"(W1 >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
+#undef MFMA_TEXT
+}
+template <int R>
+__device__ __forceinline__ float acc_fixed_read()
+{
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(R));
+    return x;
+}
+template <int R>
+__device__ __forceinline__ void acc_fixed_zero()
+{
+    asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(R));
+}
+
+// ---- vector-memory primitives.  Every VMEM operation of the pipeline is issued through inline assembly
+// and every wait on the VMEM counter is written by hand: the counter retires loads in issue order, the
+// issue order below is fixed, so "all but the N youngest operations have completed" is exact.  (Left to
+// the compiler, the waits around loop back-edges and around LDS-DMA operations collapse the prefetch
+// distance to one or two K-steps.)
+__device__ __forceinline__ v4i make_rsrc(const void* p, u32 bytes)
+{
+    const unsigned long long a = (unsigned long long)p;
+    // raw buffer: base[47:0], stride 0, num_records = bytes, word 3 = 32-bit data format
+    return (v4i){(int)(u32)a, (int)((a >> 32) & 0xFFFFu), (int)bytes, 0x00020000};
+}
+// address = rsrc.base + voff + soff + IMM (IMM < 4096); only voff + IMM is range-checked
+template <int IMM = 0, bool NT = false>
+__device__ __forceinline__ void vm_load_b128(v4i& dst, int voff, v4i rsrc, int soff)
+{
+    if(NT)      // streamed once: the line is the first to go when the L2 needs room
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4 nt" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+    else
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+}
+template <int IMM = 0>
+__device__ __forceinline__ void vm_load_b32(int& dst, int voff, v4i rsrc, int soff)
+{
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen offset:%4" : "=v"(dst) : "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory");
+}
+// global -> LDS without passing through registers: lane i's bytes land at lds_base + LDS_IMM + i * size.
+// (The hardware adds the instruction's immediate offset to the LDS address as well as to the global one, so
+// M0 is set to the target minus IMM.)  M0 cannot be named as a clobber: it is a reserved register for the compiler,
+// which neither tracks nor preserves it around inline assembly (it says so when asked to).  These helpers are sound
+// as long as the compiler's own code never uses M0 in these kernels (on gfx9 LDS instructions do not need it);
+// tests/test_build_checks.py checks on the generated code that nothing outside the inline assembly names M0.
+template <int IMM, int LDS_IMM, bool NT = false>
+__device__ __forceinline__ void vm_dma_b128(int voff, v4i rsrc, int soff, u32 lds_base)
+{
+    if(NT)      // streamed once: the line is the first to go when the L2 needs room
+        asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen offset:%4 nt lds"
+                     ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
+    else
+        asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen offset:%4 lds"
+                     ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
+}
+template <int IMM, int LDS_IMM>
+__device__ __forceinline__ void vm_dma_b32(int voff, v4i rsrc, int soff, u32 lds_base)
+{
+    asm volatile("s_add_u32 m0, %3, %5\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen offset:%4 lds"
+                 ::"v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base), "n"(IMM), "n"(LDS_IMM - IMM) : "memory", "scc");
+}
+// The same for descriptors that were just made uniform with v_readfirstlane: a vector-memory instruction must not
+// read a scalar register earlier than 5 wait states after a vector instruction wrote it, and the compiler does
+// not look into inline assembly for that (tests/test_build_checks.py scans the generated code for the pattern).
+__device__ __forceinline__ void vm_dma_b32_fresh_sgprs(int voff, v4i rsrc, u32 lds_base)
+{
+    asm volatile("s_nop 4\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
+                 ::"v"(voff), "s"(rsrc), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ u32 lds_addr_of(const void* p)
+{
+    return (u32)(unsigned long long)(__attribute__((address_space(3))) const void*)p;
+}
+// all but the N youngest VMEM operations have completed; the registers named are (re)defined here, so
+// their consumers cannot be scheduled above the wait
+template <int N>
+__device__ __forceinline__ void wait_vm_tiles(v4i& a, v4i& b, v4i& c, v4i& d)
+{
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm_scales(int& a, int& b, int& c, int& d)
+{
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_barrier()
+{
+    // own DMA writes complete (all but the N youngest VMEM ops), own LDS reads complete, then meet
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// 4x4 transpose of dwords across the four 16-lane rows of a wave: in: x[j] of lane row kb;
+// out: x[c] of lane row q holds what x[q] of lane row c held.  (permlane32_swap exchanges lanes
+// 32..63 of its first operand with lanes 0..31 of its second; permlane16_swap exchanges the odd
+// 16-lane rows of its first operand with the even rows of its second.)
+__device__ __forceinline__ void transpose4x4_rows(u32 (&x)[4])
+{
+    typedef unsigned v2u __attribute__((ext_vector_type(2)));
+    v2u t;
+    t = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false); x[0] = t.x; x[2] = t.y;
+    t = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false); x[1] = t.x; x[3] = t.y;
+    t = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false); x[0] = t.x; x[1] = t.y;
+    t = __builtin_amdgcn_permlane16_swap(x[2], x[3], false, false); x[2] = t.x; x[3] = t.y;
+}
+
+struct TileId
+{
+    int m_blk, nt, e;   // row block, weight tile, (local) expert; all wave-uniform
+    bool valid;
+};
+
+// compute units of the current device (asked once per device, then remembered)
+static inline int device_cu_count()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 256;
+    int cus = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if(cus == 0)
+    {
+        if(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        __atomic_store_n(&cached[dev], cus, __ATOMIC_RELAXED);
+    }
+    return cus;
+}
+

@@ -134,6 +134,7 @@ def fused_moe(
     stage_events=None,
     swiglu_limit=None,
     topk_reduce="store",
+    operand_staging="registers",
 ):
     """See the module docstring.  Extras beyond the reference signature: ``dtype=torch.float32`` returns
     the fp32 top-k sum without the final bf16 rounding; ``return_parts=True`` also returns the
@@ -141,7 +142,11 @@ def fused_moe(
     ``activation=ActivationType.Swiglu`` selects gpt-oss's clamped SwiGLU with ``swiglu_limit`` (default 7.0, as
     tests/contrib/moe/test_moe.py:76-81); ``topk_reduce="atomic"`` (MXFP4-activation path, row block 16 or 128,
     bf16 output) lets the down GEMM add its results into the output with packed bf16 atomics, the reference's atomic
-    variant (src/contrib/moe_gemm_mxfp4.py:1334-1398), instead of the deterministic store + reduction."""
+    variant (src/contrib/moe_gemm_mxfp4.py:1334-1398), instead of the deterministic store + reduction;
+    ``operand_staging="lds"`` (MXFP4-activation path, 256-row blocks, at most 512 experts) runs both GEMMs on the
+    eight-wave tile whose weights, too, are staged through LDS (the tile shape of the reference's prefill kernel,
+    src/contrib/moe_gemm_mxfp4.py:318-637) instead of the tiles that load weights straight into registers:
+    bit-identical results, measured slower, never chosen automatically."""
     lib = _lib.load()
     _require(activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts only")
     act = 1 if activation == ActivationType.Swiglu else 0
@@ -157,6 +162,7 @@ def fused_moe(
     _require(out_dtype in (torch.bfloat16, torch.float32), "dtype must be bfloat16 or float32", TypeError)
     _require(method in ("auto", "a4w4", "w4a16", "jit", "gluon"), "method=%r" % (method,))
     _require(topk_reduce in ("store", "atomic"), "topk_reduce=%r" % (topk_reduce,))
+    _require(operand_staging in ("registers", "lds"), "operand_staging=%r" % (operand_staging,))
 
     # weights in the plain layout (no ``is_shuffled`` mark) are re-tiled once; the scales always come e8m0-shuffled,
     # as the reference passes them (tests/contrib/moe/test_moe.py:167-189)
@@ -214,12 +220,17 @@ def fused_moe(
         _require(num_local_tokens.is_cuda and num_local_tokens.dtype == torch.int32,
                  "num_local_tokens must be an int32 scalar tensor on the GPU", TypeError)
 
+    lds_tile = operand_staging == "lds"
+    if lds_tile:
+        _require(not w4a16 and block_size_M in (None, 256) and topk_reduce == "store",
+                 "operand_staging='lds' needs the MXFP4-activation path, 256-row blocks and topk_reduce='store'")
+        bm = 256
     atomic = topk_reduce == "atomic"
     if atomic:
         _require(not w4a16 and bm in (16, 128) and out_dtype == torch.bfloat16,
                  "topk_reduce='atomic' needs the MXFP4-activation path, a row block of 16 or 128 and bf16 output")
 
-    if not return_parts and stage_events is None and not atomic:
+    if not return_parts and stage_events is None and not atomic and not lds_tile:
         # the whole layer in one library call, intermediates in one workspace: two allocations and one foreign call
         # per layer instead of a dozen of each (the host side is what bounds small layers when they are not replayed
         # from a graph)
@@ -288,10 +299,16 @@ def fused_moe(
     a2 = torch.empty(n_blk * bm, I, dtype=torch.bfloat16, device=dev) if return_parts else None
     a2_q = torch.empty(n_blk * bm, I // 2, dtype=torch.uint8, device=dev)
     a2_s = torch.empty(n_blk * bm, lib.pyhip_moe_act_scale_stride(I), dtype=torch.uint8, device=dev)
-    rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
-                                   _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
-                                   _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
-                                   _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, act, limit, stream)
+    if lds_tile:
+        rc = lib.pyhip_moe_gemm1_mxfp4_lds(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
+                                           _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
+                                           _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
+                                           _lib.dptr(a2_s), T, k, global_E, H, I, n_blk, act, limit, stream)
+    else:
+        rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
+                                       _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
+                                       _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
+                                       _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, act, limit, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
     if atomic:
@@ -306,10 +323,16 @@ def fused_moe(
         _mark("gemm2", ev)
     else:
         out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
-        rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
-                                       _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
-                                       _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
-                                       T, k, global_E, H, I, bm, n_blk, stream)
+        if lds_tile:
+            rc = lib.pyhip_moe_gemm2_mxfp4_lds(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                               _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                               _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched),
+                                               _lib.dptr(out3), T, k, global_E, H, I, n_blk, stream)
+        else:
+            rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                           _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                           _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
+                                           T, k, global_E, H, I, bm, n_blk, stream)
         _lib.check(rc, "moe_gemm2_mxfp4")
         ev = _mark("gemm2", ev)
         out = torch.empty(T, H, dtype=out_dtype, device=dev)

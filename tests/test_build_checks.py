@@ -15,21 +15,39 @@ SRC = os.path.join(ROOT, "pyhip_amd", "csrc", "moe_gemm_mxfp4.hip")
 KERNEL_RE = r"^(_Z21moe_gemm_mxfp4_kernelILi\dELi\d+ELi\dELb[01]ELb[01]EEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel"
 
 
-@pytest.fixture(scope="module")
-def gemm_asm(tmp_path_factory):
-    """the device assembly of the GEMM source, compiled once with the library's own flags"""
+WIDE_SRC = os.path.join(ROOT, "pyhip_amd", "csrc", "moe_gemm_mxfp4_wide.hip")
+WIDE_KERNEL_RE = r"^(_Z26moe_gemm_mxfp4_wide_kernelILi\dELi\dEEv8GemmArgs):[^\n]*\n(.*?)\.end_amdhsa_kernel"
+
+
+def _device_asm(tmp_path_factory, src, kernel_re):
     if shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"):
         pytest.skip("needs hipcc")
     from pyhip_amd import build
-    out = tmp_path_factory.mktemp("asm") / "gemm.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", SRC, "-o", str(out)]
+    out = tmp_path_factory.mktemp("asm") / (os.path.basename(src) + ".s")
+    cmd = [build.HIPCC] + [f for f in build.FLAGS if f not in ("-fPIC",)] + ["--cuda-device-only", "-S", src, "-o", str(out)]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout[-2000:]
     text = out.read_text()
-    kernels = re.findall(KERNEL_RE, text, re.S | re.M)
+    return text, re.findall(kernel_re, text, re.S | re.M)
+
+
+@pytest.fixture(scope="module")
+def four_wave_asm(tmp_path_factory):
+    """the device assembly of the four-wave GEMM source, compiled once with the library's own flags"""
+    text, kernels = _device_asm(tmp_path_factory, SRC, KERNEL_RE)
     assert len(kernels) == 34, ("expected (gate_up x two activations + down) x five tile heights x two load policies, "
                                 "plus the down GEMM with the atomic epilogue at two tile heights x two load policies")
     return text, kernels
+
+
+@pytest.fixture(scope="module")
+def gemm_asm(tmp_path_factory, four_wave_asm):
+    """... plus the eight-wave kernels (gate_up x two activations + down), which name their accumulators, set M0 and
+    issue vector-memory instructions by hand in the same way"""
+    text, kernels = four_wave_asm
+    wide_text, wide = _device_asm(tmp_path_factory, WIDE_SRC, WIDE_KERNEL_RE)
+    assert len(wide) == 3
+    return text + wide_text, kernels + wide
 
 
 def test_compiler_never_touches_accumulation_registers_of_fixed_tiles(gemm_asm):
@@ -114,13 +132,14 @@ def _vgprs(operand_text):
     return regs
 
 
-def test_compiler_never_copies_a_register_with_a_load_in_flight(gemm_asm):
+def test_compiler_never_copies_a_register_with_a_load_in_flight(four_wave_asm):
     """The weight tiles and weight scales are loaded by inline assembly long before they are used, and only the
     hand-written waits know when they have arrived.  That holds as long as the compiler leaves those registers
     alone: a copy it inserts (live-range splitting, a join between two instances of a loop body) would read a
     register whose load is still in flight.  Check: outside the inline-assembly regions no instruction of a GEMM
-    kernel reads or writes a register that an inline-assembly load writes to."""
-    _, kernels = gemm_asm
+    kernel reads or writes a register that an inline-assembly load writes to.  (The eight-wave kernels load nothing
+    but their weight scales into registers and copy those on purpose, after the wait that covers them.)"""
+    _, kernels = four_wave_asm
     for name, body in kernels:
         # Walk the kernel text: a register is "loaded" from the inline-assembly load that writes it until the
         # compiler's own code overwrites it with something else.  Values loaded that way are consumed by

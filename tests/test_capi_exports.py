@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.pyhip_moe_abi_version() == 5
+    assert lib.pyhip_moe_abi_version() == 6
 
 
 def test_size_helpers():
@@ -57,6 +57,9 @@ def test_argument_errors_are_reported():
     assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
     rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 48, 4, None)
     assert rc == 1 and b"block_m" in lib.pyhip_moe_last_error()
+    # the tile with both operands through LDS only exists with the sort's schedule
+    rc = lib.pyhip_moe_gemm1_mxfp4_lds(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1024, 1024, 4, 0, 0.0, None)
+    assert rc == 1 and b"schedule missing" in lib.pyhip_moe_last_error()
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -185,6 +185,10 @@ def test_tile_heights_agree_bit_for_bit(layer):
     assert torch.isfinite(outs[bms[0]].float()).all()
     for bm in bms[1:]:
         assert torch.equal(outs[bm], outs[bms[0]]), bm
+    # and so does the eight-wave 256-row tile that stages the weights through LDS as well (gpt-oss: with biases and
+    # the clamped SwiGLU in its epilogue)
+    via_lds = _run(W, hidden, tw, ti, method="a4w4", operand_staging="lds")
+    assert torch.equal(via_lds, outs[bms[0]])
 
 
 @pytest.mark.parametrize("layer", ["dsv3"], indirect=True)

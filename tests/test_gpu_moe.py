@@ -311,6 +311,11 @@ def test_swiglu_matches_oracle(method, limit, T):
         assert np.mean(err > TOL_MAX) <= 2e-3 and err.max() <= 0.1
     assert cos >= TOL_COS
     assert metrics.cosine(got, silu_ref) < 0.99                                 # and it is not SiLU
+    if method == "a4w4":
+        # the eight-wave tile with both operands through LDS has its own instance of this epilogue: same bits
+        kw = dict(w1_scale=w1s, w2_scale=w2s, bias1=b1, bias2=b2, hidden_pad=hp, intermediate_pad=ip, dtype=torch.float32,
+                  method=method, activation=ActivationType.Swiglu, swiglu_limit=limit)
+        assert torch.equal(fused_moe(L.hidden.cuda(), w1, w2, tw, ti, operand_staging="lds", **kw), out32)
 
 
 def test_prepared_weight_file_feeds_the_operator(tmp_path):
@@ -637,3 +642,41 @@ def test_more_experts_than_the_tile_schedule_holds(T, bm):
     ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4", bias1=_f(L.bias1),
                       bias2=_f(L.bias2))
     _end_to_end(_f(out32), ref, ref_a2, nflip1)
+
+
+@pytest.mark.parametrize("name,T,bias", [("mixtral_s", 700, False), ("mixtral_s", 40, True), ("longk_s", 300, True),
+                                         ("odd", 520, False), ("gptoss_s1", 260, True)])
+def test_tile_with_both_operands_through_lds(name, T, bias):
+    """operand_staging="lds": the eight-wave 256-row tile (weights and activations both by LDS-DMA, two wave rows half
+    a K-step apart) against the oracle, to the bounds of the other end-to-end cases, and bit for bit against the tiles
+    that load weights into registers.  Shapes with two to five K-groups per tile (odd counts change the parity of the
+    scale stages from tile to tile), experts with several row blocks and with a nearly empty last one."""
+    L = cases.make_layer(name, T, seed=7, bias=bias)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    b1 = None if L.bias1 is None else L.bias1.cuda()
+    b2 = None if L.bias2 is None else L.bias2.cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s, bias1=b1, bias2=b2, dtype=torch.float32, method="a4w4")
+    print(f"lds-tile case {name} T={T} bias={bias}", flush=True)
+    out_lds, parts = fused_moe(L.hidden.cuda(), w1, w2, tw, ti, operand_staging="lds", return_parts=True, **kw)
+    torch.cuda.synchronize()
+    assert parts["block_m"] == 256
+    for bm in (256, 128):
+        assert torch.equal(out_lds, fused_moe(L.hidden.cuda(), w1, w2, tw, ti, block_size_M=bm, **kw)), bm
+    w1e, w2e, ref_a2, nflip1 = _stage_checks(L, parts, 256)
+    assert w1e <= TOL_MAX and w2e <= TOL_MAX
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4",
+                      bias1=None if L.bias1 is None else _f(L.bias1), bias2=None if L.bias2 is None else _f(L.bias2))
+    _end_to_end(_f(out_lds), ref, ref_a2, nflip1)
+
+
+def test_lds_tile_rejects_what_it_does_not_serve():
+    """a down GEMM with a single K-group (inter = 512) has nothing to pipeline: the entry point says so"""
+    from pyhip_amd._lib import PyhipError
+    L = cases.make_layer("tiny", 40, seed=1)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    with pytest.raises(PyhipError, match="K >= 1024"):
+        fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, operand_staging="lds")
+    with pytest.raises(ValueError):
+        fused_moe(L.hidden.cuda(), w1, w2, tw, ti, w1_scale=w1s, w2_scale=w2s, operand_staging="lds", block_size_M=128)
