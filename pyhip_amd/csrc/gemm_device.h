@@ -169,6 +169,151 @@ struct TileId
     bool valid;
 };
 
+// ---- accumulators and epilogue of one wave's part of a tile.  A wave owns MT row groups of 16 rows x 4 weight row
+// groups (stage 1: groups 0, 1 are gate rows, 2, 3 the matching up rows); the accumulator of (weight row group j, row
+// group mt) is a[(j*MT + mt)*4 .. +3].
+template <int MT>
+__device__ __forceinline__ void gemm_zero_acc()
+{
+    static_for<16 * MT>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
+}
+// the four accumulators of row group MTI, plus bias (bias4(j) = the address of the lane's four bf16 biases of weight
+// row group j; re-read per row group to keep the epilogue's register need small)
+template <int MT, int MTI, typename B>
+__device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4], B bias4)
+{
+    static_for<4>([&](auto J) __attribute__((always_inline)) {
+        constexpr int j = decltype(J)::value, a0 = (j * MT + MTI) * 4;
+        row[j] = (v4f){acc_fixed_read<a0>(), acc_fixed_read<a0 + 1>(), acc_fixed_read<a0 + 2>(), acc_fixed_read<a0 + 3>()};
+        if(g.bias)
+        {
+            const uint2 b = *(const uint2*)bias4(j);
+            row[j][0] += bf16_bits_to_f32((uint16_t)b.x);
+            row[j][1] += bf16_bits_to_f32((uint16_t)(b.x >> 16));
+            row[j][2] += bf16_bits_to_f32((uint16_t)b.y);
+            row[j][3] += bf16_bits_to_f32((uint16_t)(b.y >> 16));
+        }
+    });
+}
+// e, nt: (local) expert and weight tile; row0: sorted position of the wave's first row; wcol: which 64 (stage 1: 32 + 32)
+// of the tile's weight rows the wave owns; meta: the sorted ids of the wave's rows, their routing weights mpad words
+// further; ma: how many of the wave's row groups hold real rows (a prefix; may be <= 0)
+template <int STAGE, int MT, int ACT, bool ATOMIC>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, int row0, int wcol, const u32* meta, int mpad,
+                                              int ma, int r, int kb)
+{
+    const int I = g.N / 2;   // stage 1 only
+    if(STAGE == 1)
+    {
+        // lane (r, kb) holds channels j*16 + kb*4 .. +3 (j = 0, 1) of row r.  After one permlane16 swap per
+        // packed dword a lane holds 8 consecutive channels: one 16 B store, 64 B contiguous per row and wave.
+        typedef unsigned v2u __attribute__((ext_vector_type(2)));
+        uint16_t* out = (uint16_t*)g.out;
+        const int chw = nt * 128 + wcol * 32;
+        auto bz = [&](int j) __attribute__((always_inline)) {
+            return g.bias + (size_t)e * g.N + (j >> 1) * I + chw + (j & 1) * 16 + kb * 4;
+        };
+        // after the swap: lane rows 0..3 hold channel offsets 0, 16, 8, 24
+        const int ch_out = chw + (kb & 1) * 16 + (kb >> 1) * 8;
+        static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
+            constexpr int mt = decltype(MTI)::value;
+            const int p = row0 + mt * 16 + r;
+            uint4 o     = make_uint4(0u, 0u, 0u, 0u);     // row groups that hold only padding store zeros
+            if(mt < ma)
+            {
+                v4f row[4];
+                gemm_fetch_row<MT, mt>(g, row, bz);
+                const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
+                u32 d[2][2];
+#pragma unroll
+                for(int j = 0; j < 2; j++)
+                {
+                    float v[4];
+#pragma unroll
+                    for(int i = 0; i < 4; i++)
+                        v[i] = !ok ? 0.f : ACT == 0 ? silu_f32(row[j][i]) * row[j + 2][i] : swiglu_f32(row[j][i], row[j + 2][i], g.limit);
+                    d[j][0] = pack_bf16x2(v[0], v[1]);
+                    d[j][1] = pack_bf16x2(v[2], v[3]);
+                }
+                v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
+                v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
+                // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
+                o = make_uint4(t0.x, t1.x, t0.y, t1.y);
+            }
+            if(out)
+                *(uint4*)(out + (size_t)p * I + ch_out) = o;
+            if(g.out_q)
+            {
+                // the wave's 32 channels of a row are exactly one MX block (8 channels in each of the four
+                // lane rows): block maximum across the lane rows, then the same arithmetic as the stand-alone
+                // quantiser (moe_quant.hip) on the bf16-rounded values, so both paths agree bit for bit
+                u32 am = amax15(amax15(amax15(amax15(0u, o.x), o.y), o.z), o.w);
+                v2u s16 = __builtin_amdgcn_permlane16_swap(am, am, false, false);
+                am      = s16.x > s16.y ? s16.x : s16.y;
+                v2u s32 = __builtin_amdgcn_permlane32_swap(am, am, false, false);
+                am      = s32.x > s32.y ? s32.x : s32.y;
+                const u32 e8 = mx_scale_byte(am);
+                *(u32*)(g.out_q + (size_t)p * (I / 2) + ch_out / 2) = cvt8(o, mx_inv_scale(e8));
+                if(kb == 0)
+                {
+                    const int blk = nt * 4 + wcol, jb = blk & 15;      // scale byte: see moe_quant.hip
+                    g.out_s[(size_t)p * g.OSK + (blk & ~15) + (jb & 3) * 4 + (jb >> 2)] = (uint8_t)e8;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
+        });
+    }
+    else
+    {
+        // lane (r, kb) holds channels j*16 + kb*4 .. +3 (j = 0..3) of row r.  A 4x4 transpose across the
+        // four lane rows gives every lane 16 consecutive channels: 32 B stores, 128 B contiguous per row.
+        uint16_t* out = (uint16_t*)g.out;
+        const int chw = nt * 256 + wcol * 64;
+        auto bz = [&](int j) __attribute__((always_inline)) { return g.bias + (size_t)e * g.N + chw + j * 16 + kb * 4; };
+        static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
+            constexpr int mt = decltype(MTI)::value;
+            if(mt >= ma)
+                return;
+            v4f row[4];
+            gemm_fetch_row<MT, mt>(g, row, bz);
+            const u32 id   = meta[mt * 16 + r];
+            const float rw = __builtin_bit_cast(float, meta[mpad + mt * 16 + r]);
+            const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
+            const bool ok = slot < g.topk && tok < g.T;
+            u32 lo[4], hi[4];
+#pragma unroll
+            for(int j = 0; j < 4; j++)
+            {
+                lo[j] = pack_bf16x2(row[j][0] * rw, row[j][1] * rw);
+                hi[j] = pack_bf16x2(row[j][2] * rw, row[j][3] * rw);
+            }
+            transpose4x4_rows(lo);
+            transpose4x4_rows(hi);
+            // lane row q now holds channels q*16 + c*4 .. +3 in (lo[c], hi[c])
+            if(ok && !ATOMIC)
+            {
+                // (plain stores: marked non-temporal they cost the down GEMM 5 % and the reduction, which then finds
+                // nothing of out3 in the last-level cache, another 4 %)
+                uint4* dst = (uint4*)(out + ((size_t)tok * g.topk + slot) * g.N + chw + kb * 16);
+                dst[0]     = make_uint4(lo[0], hi[0], lo[1], hi[1]);
+                dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
+            }
+            if(ok && ATOMIC)
+            {
+                typedef short v2s __attribute__((ext_vector_type(2)));
+                auto* dst = (__attribute__((address_space(1))) v2s*)(out + (size_t)tok * g.N + chw + kb * 16);
+#pragma unroll
+                for(int c = 0; c < 4; c++)
+                {
+                    __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c, __builtin_bit_cast(v2s, lo[c]));
+                    __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c + 1, __builtin_bit_cast(v2s, hi[c]));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
+        });
+    }
+}
+
 // compute units of the current device (asked once per device, then remembered)
 static inline int device_cu_count()
 {
