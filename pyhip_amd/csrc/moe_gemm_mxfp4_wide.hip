@@ -139,10 +139,11 @@ __global__ void __launch_bounds__(WIDE_THREADS) moe_gemm_mxfp4_wide_kernel(GemmA
         t.valid = true;
     };
 
-    // ---- load side.  Descriptors and per-lane offsets exist twice: `_c` for the tile whose K-steps are being computed
-    // (the DMAs of its K-step 4*ks+3 are issued during K-step 4*ks), `_p` for the K-group that is being prefetched (the
-    // next one of this tile, or the first one of the workgroup's next tile).  A tile that does not exist is prefetched
-    // with offsets beyond every buffer: the hardware drops the accesses, the instruction stream stays the same.
+    // ---- load side.  `_p`: descriptors and lane offsets of the K-group that is being prefetched (the next one of this
+    // tile, or the first one of the workgroup's next tile): every weight DMA uses them (weights run a whole K-group
+    // ahead).  The activation DMAs run two K-steps ahead, so those of K-steps 2 and 3 of a K-group still belong to the
+    // tile being computed: its lane offsets are kept in `a_c`.  A tile that does not exist is prefetched with offsets
+    // beyond every buffer: the hardware drops the accesses, the instruction stream stays the same.
     constexpr u32 OOB = 0xFFFF0000u;
     const int dma_row   = lane >> 2;
     const int dma_chunk = (lane & 3) ^ ((lane >> 3) & 3);
