@@ -75,15 +75,21 @@ def test_pad_layer_weights_is_exact():
 
 
 def test_row_block_heuristic():
-    """smallest of 16 / 32 / 64 / 128 that holds twice the mean rows per expert"""
+    """16 rows below 4 expected rows per expert, 32 below 12, 64 up to 32, 128 above"""
     from pyhip_amd.fused_moe import pick_block_m
     assert pick_block_m(16, 8, 256) == 16            # 0.5 rows per expert
-    assert pick_block_m(256, 8, 256) == 16           # 8
-    assert pick_block_m(512, 8, 256) == 32           # 16
+    assert pick_block_m(96, 8, 256) == 16            # 3
+    assert pick_block_m(128, 8, 256) == 32           # 4
+    assert pick_block_m(256, 8, 256) == 32           # 8
+    assert pick_block_m(384, 8, 256) == 64           # 12
+    assert pick_block_m(512, 8, 256) == 64           # 16
     assert pick_block_m(1024, 8, 256) == 64          # 32
+    assert pick_block_m(1056, 8, 256) == 128         # 33
     assert pick_block_m(2048, 8, 256) == 128         # 64
     assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
-    assert pick_block_m(1, 2, 8) == 16 and pick_block_m(4096, 2, 8) == 128
+    # few experts: the smallest tile that holds twice the mean
+    assert pick_block_m(1, 2, 8) == 16 and pick_block_m(32, 2, 8) == 16 and pick_block_m(64, 2, 8) == 32
+    assert pick_block_m(128, 2, 8) == 64 and pick_block_m(4096, 2, 8) == 128
     # the 256-row tile: 120..192 rows per expert and a long K loop
     assert pick_block_m(4096, 8, 256, 7168) == 256 and pick_block_m(6144, 8, 256, 7168) == 256
     assert pick_block_m(3584, 8, 256, 7168) == 128 and pick_block_m(7168, 8, 256, 7168) == 128
