@@ -143,7 +143,7 @@ def time_point(torch, fused_moe, W, shape, tokens, steps, warmup, block_m, metho
     cfg = workloads.SHAPES[shape]
     Hp = cfg["H"] + W["hidden_pad"]
     w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(tokens, cfg["k"], cfg["E"], Hp))
-    bm = block_m or pick_block_m(tokens, cfg["k"], cfg["E"], Hp)
+    bm = block_m or pick_block_m(tokens, cfg["k"], cfg["E"], Hp, w4a16)
     return dict(wall_ms=wall_ms, median_ms=q(0.5), q1_ms=q(0.25), q3_ms=q(0.75), work=work, hidden=hidden,
                 topk_w=topk_w, topk_ids=topk_ids, out=out, method="w4a16" if w4a16 else "a4w4",
                 block_m=min(bm, 64) if w4a16 else bm, weight_copies=len(sets), calls_per_batch=reps)

@@ -240,9 +240,9 @@ int pyhip_moe_zero_fill(void* p, int64_t bytes, pyhip_stream_t stream);
  *   block_m       the row block: 16/32/64, with MXFP4 activations also 128/256
  *   w4a16         0 = MXFP4 activations (pyhip_moe_gemm*_mxfp4), 1 = bf16 activations (pyhip_moe_gemm*_w4a16)
  * pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 give the choices the reference's operator makes inside fused_moe
- * (block_size_M=None, method="auto": src/contrib/fused_moe.py:128-155) as this library makes them; with w4a16 the
- * row block is at most 64. */
-int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int hidden);
+ * (block_size_M=None, method="auto": src/contrib/fused_moe.py:128-155) as this library makes them (the row block for
+ * the kernel family given by w4a16; with bf16 activations it is at most 64). */
+int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int hidden, int w4a16);
 int pyhip_moe_pick_w4a16(int64_t tokens, int topk, int experts, int hidden);
 int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, int experts, int hidden, int inter, int block_m,
                                           int w4a16);

@@ -21,7 +21,7 @@ SIGNATURES = {
     "pyhip_moe_sorting_workspace_bytes": (_L, [_L, _I, _I]),
     "pyhip_moe_schedule_words": (_L, [_I]),
     "pyhip_moe_sorting": (_I, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _P]),
-    "pyhip_moe_pick_block_m": (_I, [_L, _I, _I, _I]),
+    "pyhip_moe_pick_block_m": (_I, [_L, _I, _I, _I, _I]),
     "pyhip_moe_pick_w4a16": (_I, [_L, _I, _I, _I]),
     "pyhip_moe_zero_fill": (_I, [_P, _L, _P]),
     "pyhip_moe_forward_workspace_bytes": (_L, [_L, _I, _I, _I, _I, _I, _I]),

@@ -79,7 +79,7 @@ Layout make_layout(int64_t T, int k, int E, int H, int I, int bm, int w4a16)
 
 // The choices pyhip_amd/fused_moe.py makes for method="auto" and block_size_M=None (pick_block_m, pick_w4a16; the
 // measurements behind them are quoted there), for callers that bind the library without the Python layer.
-extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int hidden)
+extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int hidden, int w4a16)
 {
     const double est = (double)tokens * topk / (experts > 0 ? experts : 1);      // routed rows per expert, on average
     // The tile is chosen from the AVERAGE load, which is all that is known before the sort has run, with room for routers
@@ -92,7 +92,9 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
     // With a handful of experts (Mixtral: 8) every expert gets many rows, the loads are even in relative terms, and the
     // number of tiles is what such layers are short of: "twice the mean" stays (Mixtral shape, 32 tokens: 0.134 ms with
     // 16-row blocks, 0.158 with 32).
-    if(experts < 32)
+    // The same holds for the bf16-activation kernels, whose 32-row tile already halves the waves per SIMD (DeepSeek-V3
+    // shape, 128 tokens, forced: gate_up 623 us with 16-row blocks, 761 with 32); their row block is at most 64.
+    if(experts < 32 || w4a16)
     {
         for(int bm = 16; bm <= 64; bm *= 2)
             if(2 * est <= bm)
@@ -107,6 +109,8 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
         if(est <= 32)
             return 64;
     }
+    if(w4a16)
+        return 64;
     return (hidden >= 6144 && est >= 120 && est <= 192) ? 256 : 128;
 }
 

@@ -65,7 +65,7 @@ def _shuffled_u8(w):
     return out
 
 
-def pick_block_m(tokens, topk, experts, hidden=0):
+def pick_block_m(tokens, topk, experts, hidden=0, w4a16=False):
     """M-tile (= sort block size), from the expected rows per expert ``est = tokens * topk / experts``: 16 rows below 4,
     32 below 12, 64 up to 32, 128 above (layers with fewer than 32 experts: the smallest of 16 / 32 / 64 that holds
     twice ``est``).  Every extra row block of an expert streams the expert's weights once more,
@@ -80,7 +80,7 @@ def pick_block_m(tokens, topk, experts, hidden=0):
     tile one, read with non-temporal loads.  Its long epilogue only pays with a long K loop: DS-V3 (hidden 7168)
     T = 4096 / 5120 / 6144: 1.55 / 1.65 / 1.72 ms against 1.69 / 2.09 / 1.92 ms; the gpt-oss, Qwen3 and Mixtral shapes
     (hidden 3072 / 4096) lose 4-13 % with it at the same rows per expert."""
-    return int(_lib.load().pyhip_moe_pick_block_m(tokens, topk, experts, hidden))
+    return int(_lib.load().pyhip_moe_pick_block_m(tokens, topk, experts, hidden, 1 if w4a16 else 0))
 
 
 def pick_w4a16(tokens, topk, experts, hidden):
@@ -207,7 +207,7 @@ def fused_moe(
     topk_weight = topk_weight.to(torch.float32).contiguous()
     # "auto" (and the reference's "jit" / "gluon", which name its own back ends): see pick_w4a16
     w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, k, global_E, H))
-    bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E, H)
+    bm = block_size_M if block_size_M is not None else pick_block_m(T, k, global_E, H, w4a16)
     if w4a16:
         bm = min(bm, 64)
     if bias1 is not None:
@@ -382,7 +382,7 @@ def fused_moe_routed(hidden_states, w1, w2, gating_output, topk, renormalize=Tru
     if expert_mask is not None:
         expert_mask = expert_mask.to(device=dev, dtype=torch.int32).contiguous()
     w4a16 = method == "w4a16" or (method != "a4w4" and pick_w4a16(T, topk, global_E, H))
-    bm = block_size_M if block_size_M is not None else pick_block_m(T, topk, global_E, H)
+    bm = block_size_M if block_size_M is not None else pick_block_m(T, topk, global_E, H, w4a16)
     if w4a16:
         bm = min(bm, 64)
     if bias1 is not None:

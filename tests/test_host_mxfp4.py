@@ -87,6 +87,9 @@ def test_row_block_heuristic():
     assert pick_block_m(1056, 8, 256) == 128         # 33
     assert pick_block_m(2048, 8, 256) == 128         # 64
     assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
+    # the bf16-activation kernels: twice the mean, at most 64 rows
+    assert pick_block_m(128, 8, 256, 7168, True) == 16 and pick_block_m(256, 8, 256, 7168, True) == 16
+    assert pick_block_m(512, 8, 256, 7168, True) == 32 and pick_block_m(8192, 8, 256, 7168, True) == 64
     # few experts: the smallest tile that holds twice the mean
     assert pick_block_m(1, 2, 8) == 16 and pick_block_m(32, 2, 8) == 16 and pick_block_m(64, 2, 8) == 32
     assert pick_block_m(128, 2, 8) == 64 and pick_block_m(4096, 2, 8) == 128
@@ -116,5 +119,6 @@ def test_library_makes_the_same_choices():
     lib = _lib.load()
     for E, k, H in ((8, 2, 1024), (8, 2, 4096), (128, 4, 3072), (128, 8, 4096), (256, 8, 7168), (12, 3, 1536)):
         for T in list(range(1, 70)) + [96, 128, 200, 256, 500, 512, 1000, 1024, 2048, 3072, 3840, 4096, 5000, 6144, 6145, 8192, 32768]:
-            assert lib.pyhip_moe_pick_block_m(T, k, E, H) == pick_block_m(T, k, E, H), (T, k, E, H)
+            for w4 in (0, 1):
+                assert lib.pyhip_moe_pick_block_m(T, k, E, H, w4) == pick_block_m(T, k, E, H, bool(w4)), (T, k, E, H, w4)
             assert bool(lib.pyhip_moe_pick_w4a16(T, k, E, H)) == pick_w4a16(T, k, E, H), (T, k, E, H)
