@@ -41,14 +41,34 @@ struct GemmArgs
 // inside this statement, so that nothing else about the generated code changes: the pair costs more issue time in
 // full tiles than the skipped MFMAs save elsewhere: DeepSeek-V3 shape, 8192 tokens, where a fifth of the row groups
 // are padding: gate_up 1.30 -> 1.38 ms; Mixtral shape, 4096 tokens, no padding: 0.477 -> 0.503 ms.)
+// (The 288-row tile has 72 accumulator tiles, eight more than the 256 accumulation registers hold: those of weight row
+// group 3 and row groups ACC_SPILL_MT0 .. 17 are ordinary vectors, handed in as `xacc`.)
+#define ACC_SPILL_MT0 10
+template <int MT, int MTI>
+constexpr bool acc_in_vgprs() { return (3 * MT + MTI) * 4 >= 256; }
 template <int U, int MTI, int MT>
-__device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale)
+__device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale,
+                                               v4f* xacc = nullptr)
 {
     constexpr int A0 = (0 * MT + MTI) * 4, A1 = (1 * MT + MTI) * 4, A2 = (2 * MT + MTI) * 4, A3 = (3 * MT + MTI) * 4;
+    static_assert(A2 + 3 < 256, "only weight row group 3 may overflow the accumulation registers");
     constexpr int W0 = (U & 1) * 2 + 0, W1 = (U & 1) * 2 + 1;       // weight-scale byte: (kt%2)*2 + (row%32)/16
 #define MFMA_TEXT(ACC, ACCE, W, WS, WL, WH)                                                                            \
     "v_mfma_scale_f32_16x16x128_f8f6f4 a[%[" #ACC "]:%[" #ACCE "]], %[" #W "], %[a], a[%[" #ACC "]:%[" #ACCE "]], %[" #WS  \
     "], %[as] op_sel:[%[" #WL "],%[al],0] op_sel_hi:[%[" #WH "],%[ah],0] cbsz:4 blgp:4\n\t"
+    if constexpr(acc_in_vgprs<MT, MTI>())
+    {
+        asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
+                     MFMA_TEXT(c2, e2, w2, s23, x0l, x0h)
+                     "v_mfma_scale_f32_16x16x128_f8f6f4 %[xa], %[w3], %[a], %[xa], %[s23], %[as] op_sel:[%[x1l],%[al],0] "
+                     "op_sel_hi:[%[x1h],%[ah],0] cbsz:4 blgp:4\n\t"
+                     : [xa] "+v"(*xacc)
+                     : [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3), [c2] "n"(A2), [e2] "n"(A2 + 3),
+                       [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
+                       [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [x0l] "n"(W0 & 1), [x0h] "n"(W0 >> 1),
+                       [x1l] "n"(W1 & 1), [x1h] "n"(W1 >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
+    }
+    else
     asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
                  MFMA_TEXT(c2, e2, w2, s23, x0l, x0h) MFMA_TEXT(c3, e3, w3, s23, x1l, x1h)
                  :
@@ -173,18 +193,25 @@ struct TileId
 // groups (stage 1: groups 0, 1 are gate rows, 2, 3 the matching up rows); the accumulator of (weight row group j, row
 // group mt) is a[(j*MT + mt)*4 .. +3].
 template <int MT>
-__device__ __forceinline__ void gemm_zero_acc()
+__device__ __forceinline__ void gemm_zero_acc(v4f* xacc = nullptr)
 {
-    static_for<16 * MT>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
+    static_for<(16 * MT < 256 ? 16 * MT : 256)>([&](auto R) __attribute__((always_inline)) { acc_fixed_zero<decltype(R)::value>(); });
+    if constexpr(16 * MT > 256)
+#pragma unroll
+        for(int i = 0; i < (16 * MT - 256) / 4; i++)
+            xacc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 }
 // the four accumulators of row group MTI, plus bias (bias4(j) = the address of the lane's four bf16 biases of weight
 // row group j; re-read per row group to keep the epilogue's register need small)
 template <int MT, int MTI, typename B>
-__device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4], B bias4)
+__device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4], B bias4, const v4f* xacc)
 {
     static_for<4>([&](auto J) __attribute__((always_inline)) {
         constexpr int j = decltype(J)::value, a0 = (j * MT + MTI) * 4;
-        row[j] = (v4f){acc_fixed_read<a0>(), acc_fixed_read<a0 + 1>(), acc_fixed_read<a0 + 2>(), acc_fixed_read<a0 + 3>()};
+        if constexpr(a0 >= 256)
+            row[j] = xacc[MTI - ACC_SPILL_MT0];
+        else
+            row[j] = (v4f){acc_fixed_read<a0>(), acc_fixed_read<a0 + 1>(), acc_fixed_read<a0 + 2>(), acc_fixed_read<a0 + 3>()};
         if(g.bias)
         {
             const uint2 b = *(const uint2*)bias4(j);
@@ -200,7 +227,7 @@ __device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4],
 // further; ma: how many of the wave's row groups hold real rows (a prefix; may be <= 0)
 template <int STAGE, int MT, int ACT, bool ATOMIC>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, int row0, int wcol, const u32* meta, int mpad,
-                                              int ma, int r, int kb)
+                                              int ma, int r, int kb, const v4f* xacc = nullptr)
 {
     const int I = g.N / 2;   // stage 1 only
     if(STAGE == 1)
@@ -222,7 +249,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
             if(mt < ma)
             {
                 v4f row[4];
-                gemm_fetch_row<MT, mt>(g, row, bz);
+                gemm_fetch_row<MT, mt>(g, row, bz, xacc);
                 const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
                 u32 d[2][2];
 #pragma unroll
@@ -275,7 +302,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
             if(mt >= ma)
                 return;
             v4f row[4];
-            gemm_fetch_row<MT, mt>(g, row, bz);
+            gemm_fetch_row<MT, mt>(g, row, bz, xacc);
             const u32 id   = meta[mt * 16 + r];
             const float rw = __builtin_bit_cast(float, meta[mpad + mt * 16 + r]);
             const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);

@@ -111,7 +111,17 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
     }
     if(w4a16)
         return 64;
-    return (hidden >= 6144 && est >= 120 && est <= 192) ? 256 : 128;
+    // Prefill sizes: 128 rows, except where a taller tile lets nearly every expert fit ONE row block, so that each weight
+    // tile is read once instead of two or three times.  The 256- and 288-row tiles run one wave per SIMD and have a long
+    // epilogue, which only pays with a long K loop (hidden >= 6144); the gpt-oss, Qwen3 and Mixtral shapes (hidden 3072 /
+    // 4096) lose 4-13 % with them at the same rows per expert.  DeepSeek-V3 shape, whole layer, ms, tiles of 128 / 256 /
+    // 288 rows: 208 rows per expert 1.94 / 1.85 / 1.87; 224: 2.07 / 1.93 / 1.93; 240: 2.09 / 2.05 / 1.97; 256 (8192 tokens):
+    // 2.29 / 2.69 / 2.06; 264: 2.44 / 3.05 / 2.11; 272: 2.49 / 3.31 / 2.39; 288: 2.57 / 3.53 / 2.97.
+    if(hidden >= 6144 && est >= 120 && est <= 224)
+        return 256;
+    if(hidden >= 6144 && est > 224 && est <= 276)
+        return 288;
+    return 128;
 }
 
 extern "C" int pyhip_moe_pick_w4a16(int64_t tokens, int topk, int experts, int hidden)
@@ -154,8 +164,9 @@ static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, cons
     PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && w2 && w2_scale && topk_ids && topk_weights && out,
                   "moe_forward: null pointer");
     PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0 && hidden > 0 && inter > 0, "moe_forward: bad sizes");
-    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || ((block_m == 128 || block_m == 256) && !w4a16),
-                  "moe_forward: block_m=%d (16/32/64, and 128/256 with MXFP4 activations)", block_m);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 ||
+                      ((block_m == 128 || block_m == 256 || block_m == 288) && !w4a16),
+                  "moe_forward: block_m=%d (16/32/64, and 128/256/288 with MXFP4 activations)", block_m);
     PYHIP_REQUIRE(!w4a16 || hidden_row_stride == hidden, "moe_forward: the bf16-activation kernels need contiguous rows");
     const Layout l = make_layout(tokens, topk, experts, hidden, inter, block_m, w4a16);
     PYHIP_REQUIRE(workspace && workspace_bytes >= l.total && ((uintptr_t)workspace % 256) == 0,

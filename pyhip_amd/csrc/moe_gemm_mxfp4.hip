@@ -47,13 +47,20 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     constexpr int BM    = MT * 16;
     // The accumulators live in the accumulation registers a0 .. a[16*MT-1], named by hand in the instruction text
     // (mfma_row_group); the clobber reserves that range for the kernel.
-    if constexpr(MT == 16) asm volatile("" ::: "a0", "a255");
+    if constexpr(MT >= 16) asm volatile("" ::: "a0", "a255");
     if constexpr(MT == 8) asm volatile("" ::: "a0", "a127");
     if constexpr(MT == 4) asm volatile("" ::: "a0", "a63");
     if constexpr(MT == 2) asm volatile("" ::: "a0", "a31");
     if constexpr(MT == 1) asm volatile("" ::: "a0", "a15");
     constexpr int NA    = (MT + 3) / 4;       // activation row groups DMA'd per wave
-    constexpr int SLOTS = NA * 4;             // row-group slots per LDS stage (slots >= MT are never read)
+    // The 288-row tile (MT = 18) is the largest that fits the CU at all: its two activation stages take 144 of the 160 KB
+    // of LDS.  It therefore has exactly MT slots per stage (the DMA operations of the two slots that do not exist go to
+    // a dummy area), a ring of two tiles' sorted ids instead of three (filled one K-group later, see meta_on), reads
+    // the schedule from global memory with scalar loads instead of keeping it in LDS, and keeps the accumulator tiles
+    // that the 256 accumulation registers do not hold in ordinary registers (xacc).
+    constexpr bool TALL = MT == 18;
+    constexpr int SLOTS = TALL ? MT : NA * 4;  // row-group slots per LDS stage (slots >= MT are never read)
+    constexpr int MR    = TALL ? 2 : 3;        // tiles in the ring of sorted ids / routing weights
     constexpr int NID   = (BM + 63) / 64;     // DMA ops that bring one tile's sorted ids (same for weights)
     constexpr int MPAD  = NID * 64;           // words per meta array
     constexpr int NM    = (2 * NID + 3) / 4;  // meta DMA ops per wave and K-group (same count in every wave)
@@ -67,11 +74,11 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     __shared__ __attribute__((aligned(16))) uint8_t lds_a1[4 * SLOTS * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t lds_s0[SLOTS * 256];
     __shared__ __attribute__((aligned(16))) uint8_t lds_s1[SLOTS * 256];
-    __shared__ u32 lds_meta[3][2 * MPAD];     // per tile: sorted ids | routing weights; ring of 3 tiles
-    __shared__ u32 lds_dummy[64];             // where the zeros of switched-off meta DMA operations land
-    constexpr int SCHED_E = MT == 1 ? SCHED_E_MAX_16 : SCHED_E_MAX;
+    __shared__ u32 lds_meta[MR][2 * MPAD];    // per tile: sorted ids | routing weights; ring of MR tiles
+    __shared__ __attribute__((aligned(16))) u32 lds_dummy[TALL ? 256 : 64];   // where switched-off DMA operations put their zeros
+    constexpr int SCHED_E = TALL ? 0 : MT == 1 ? SCHED_E_MAX_16 : SCHED_E_MAX;
     __shared__ u32 lds_pre[SCHED_E + 1];      // the schedule: row blocks before every expert (and their total),
-    __shared__ u32 lds_lid[SCHED_E];          //   local id of every expert
+    __shared__ u32 lds_lid[SCHED_E + 1];      //   local id of every expert
 
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);   // wave-uniform: keeps descriptors and LDS bases scalar
@@ -94,7 +101,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     u32 q                 = blockIdx.x >> 3;
     u32 q_end             = 0;
     int ei                = 0;                        // cursor into the expert list (q only grows)
-    if(persistent)
+    if(persistent && !TALL)
     {
         for(int i = tid; i <= g.E; i += GEMM_THREADS)
         {
@@ -105,13 +112,30 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         __syncthreads();
     }
     auto uni = [](u32 v) __attribute__((always_inline)) { return (u32)__builtin_amdgcn_readfirstlane((int)v); };
+    // the schedule: row blocks before expert i (i = E: their total) and the local id of expert i; from LDS, or (288-row
+    // tile) from global memory through the scalar cache: uniform addresses, a handful of reads per tile
+    // (the constant address space is what makes the compiler pick scalar loads: a vector load would come with a wait on
+    // the vector-memory counter, which in this pipeline means waiting for every prefetch in flight)
+    typedef const __attribute__((address_space(4))) u32* sched_ptr;
+    auto sched_pre = [&](int i) __attribute__((always_inline)) -> u32 {
+        if constexpr(TALL)
+            return ((sched_ptr)(unsigned long long)g.sched)[i];
+        else
+            return uni(lds_pre[i]);
+    };
+    auto sched_lid = [&](int i) __attribute__((always_inline)) -> u32 {
+        if constexpr(TALL)
+            return ((sched_ptr)(unsigned long long)g.sched)[g.E + 1 + i];
+        else
+            return uni(lds_lid[i]);
+    };
     auto uni4 = [](v4i v) __attribute__((always_inline)) {
         return (v4i){__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y),
                      __builtin_amdgcn_readfirstlane(v.z), __builtin_amdgcn_readfirstlane(v.w)};
     };
     if(persistent)
     {
-        const u32 tiles = uni(lds_pre[g.E]) * (u32)g.n_tiles;
+        const u32 tiles = sched_pre(g.E) * (u32)g.n_tiles;
         const u32 chunk = (tiles + 7u) >> 3;
         // (Every workgroup of the launch takes part, also when the last round of an XCD's run is nearly empty.  Letting only
         // as many take part as make the rounds even (113 tiles on 96 workgroups: 57 with two tiles each) was measured and is
@@ -126,7 +150,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             while(lo < hi)
             {
                 const int mid = (lo + hi) >> 1;
-                if(uni(lds_pre[mid + 1]) * (u32)g.n_tiles > q)
+                if(sched_pre(mid + 1) * (u32)g.n_tiles > q)
                     hi = mid;
                 else
                     lo = mid + 1;
@@ -140,14 +164,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         {
             if(q >= q_end)
                 return;
-            while(q >= uni(lds_pre[ei + 1]) * (u32)g.n_tiles)
+            while(q >= sched_pre(ei + 1) * (u32)g.n_tiles)
                 ei++;
-            const u32 p0    = uni(lds_pre[ei]);
-            const u32 nb    = uni(lds_pre[ei + 1]) - p0;
+            const u32 p0    = sched_pre(ei);
+            const u32 nb    = sched_pre(ei + 1) - p0;
             const u32 local = q - p0 * (u32)g.n_tiles;
             t.nt            = (int)(local / nb);
             t.m_blk         = (int)(p0 + (local - (u32)t.nt * nb));
-            t.e             = (int)uni(lds_lid[ei]);
+            t.e             = (int)sched_lid(ei);
             q += qstride;
         }
         else
@@ -264,15 +288,27 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // 1 KB block of a (row group, K-step) lands in MFMA operand order; 5*NA VMEM ops per wave.
     const u32 lds_a[2] = {lds_addr_of(lds_a0 + wave * 1024), lds_addr_of(lds_a1 + wave * 1024)};
     const u32 lds_s[2] = {lds_addr_of(lds_s0 + wave * 256), lds_addr_of(lds_s1 + wave * 256)};
+    // (288-row tile: the last of a wave's five slots, wave + 16, only exists for waves 0 and 1; the operations of the
+    // other two waves, whose lane offsets are out of range anyway, put their zeros into the dummy area.  LDS_IMM is the
+    // offset the DMA helper adds to the base it is given.)
+    const bool last_slot_ok = !TALL || wave + 4 * (NA - 1) < MT;
+    const u32 lds_dummy_a   = lds_addr_of(lds_dummy);
+    auto slot_base = [&](auto II, auto IMM, u32 normal) __attribute__((always_inline)) -> u32 {
+        if constexpr(TALL && decltype(II)::value == NA - 1)
+            return last_slot_ok ? normal : lds_dummy_a - (u32)decltype(IMM)::value;
+        else
+            return normal;
+    };
     auto dma_group = [&](auto S, int ks) __attribute__((always_inline)) {
         constexpr int s = decltype(S)::value;
         static_for<NA>([&](auto II) __attribute__((always_inline)) {
             constexpr int i = decltype(II)::value;
             static_for<4>([&](auto U) __attribute__((always_inline)) {
                 constexpr int u = decltype(U)::value;
-                vm_dma_b128<u * 64, (u * SLOTS + 4 * i) * 1024>(a_off[i], ars, ks * 256, lds_a[s]);
+                constexpr int imm = (u * SLOTS + 4 * i) * 1024;
+                vm_dma_b128<u * 64, imm>(a_off[i], ars, ks * 256, slot_base(II, std::integral_constant<int, imm>{}, lds_a[s]));
             });
-            vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, ks * 16, lds_s[s]);
+            vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, ks * 16, slot_base(II, std::integral_constant<int, 4 * i * 256>{}, lds_s[s]));
         });
     };
     v4i wf[4][4];
@@ -300,9 +336,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     };
 
     // accumulators and epilogue: gemm_device.h
-    auto zero_acc = [&]() __attribute__((always_inline)) { gemm_zero_acc<MT>(); };
+    v4f xacc[TALL ? MT - ACC_SPILL_MT0 : 1];      // the accumulator tiles beyond the accumulation registers (288-row tile)
+    auto zero_acc = [&]() __attribute__((always_inline)) { gemm_zero_acc<MT>(xacc); };
     auto epilogue = [&](const TileId& t, const u32* meta, int ma_t) __attribute__((always_inline)) {
-        gemm_epilogue<STAGE, MT, ACT, ATOMIC>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb);
+        gemm_epilogue<STAGE, MT, ACT, ATOMIC>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
     };
 
     // ---------------------------------------------------------------- pipeline
@@ -310,7 +347,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     decode(cur);
     if(!cur.valid)
         return;
-    int mb = 0;                                   // meta buffer of the current tile (ring of 3)
+    int mb = 0;                                   // meta buffer of the current tile (ring of MR)
     setup_load(cur, g.sorted_ids + (size_t)cur.m_blk * BM);
     int ma     = count_groups(g.sorted_ids + (size_t)cur.m_blk * BM);   // active row groups of the current tile
     int ma_nxt = ma;                                                    // ... and of the next one
@@ -330,7 +367,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         constexpr int p  = decltype(P)::value;    // parity of the global K-group count: LDS stage / scale registers
         const bool last     = ks == KS - 1;
         const int kpre      = last ? 0 : ks + 1;  // K-group that is prefetched now (of the next tile when last)
-        const int mb_nxt    = mb == 2 ? 0 : mb + 1;
+        const int mb_nxt    = mb == MR - 1 ? 0 : mb + 1;
         // (0) first K-group of a tile: ids/weights of the NEXT tile into the meta ring (two tiles ahead of the
         //     slot any wave can still be reading in its epilogue)
         // (1) descriptors of what this K-group prefetches: the next K-group of this tile, or K-group 0 of the
@@ -345,7 +382,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             else
                 setup_null();
         }
-        const bool meta_on = ks == 0 && nxt.valid;
+        // (with a ring of two the slot still belongs to the previous tile, whose epilogue a slower wave may not have
+        // finished before the barrier that ends this tile's first K-group: the fetch waits for the second K-group)
+        const bool meta_on = ks == (TALL ? 1 : 0) && nxt.valid;
         const v4i rid = make_rsrc(g.sorted_ids + (size_t)nxt.m_blk * BM, BM * 4);
         const v4i rwt = make_rsrc(g.sorted_w + (size_t)nxt.m_blk * BM, BM * 4);
         // prefetch operation K of this K-group (0 <= K < NPF)
@@ -367,10 +406,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             else if constexpr(k < NM + 5 * NA)
             {
                 constexpr int i = (k - NM) / 5, sub = (k - NM) % 5;
+                using II = std::integral_constant<int, i>;
                 if constexpr(sub < 4)
-                    vm_dma_b128<sub * 64, (sub * SLOTS + 4 * i) * 1024>(a_off[i], ars, kpre * 256, lds_a[p ^ 1]);
+                {
+                    constexpr int imm = (sub * SLOTS + 4 * i) * 1024;
+                    vm_dma_b128<sub * 64, imm>(a_off[i], ars, kpre * 256, slot_base(II{}, std::integral_constant<int, imm>{}, lds_a[p ^ 1]));
+                }
                 else
-                    vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, kpre * 16, lds_s[p ^ 1]);
+                    vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, kpre * 16, slot_base(II{}, std::integral_constant<int, 4 * i * 256>{}, lds_s[p ^ 1]));
             }
             else
             {
@@ -418,8 +461,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 const int asc = asc_all[mt];
                 __builtin_amdgcn_sched_barrier(0);
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
-                                          w_sc[p][2 + (u >> 1)], asc);
+                if constexpr(acc_in_vgprs<MT, mt>())
+                    mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
+                                              w_sc[p][2 + (u >> 1)], asc, &xacc[mt - ACC_SPILL_MT0]);
+                else
+                    mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
+                                              w_sc[p][2 + (u >> 1)], asc);
                 // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
                 // issue overlaps the matrix pipeline instead of preceding it
                 if constexpr(u == 0)
@@ -487,9 +534,11 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
         return rc;
     }
     unsigned nwg = (unsigned)(g.n_tiles * g.n_blk);
-    if(g.K < 1024 || g.E > (block_m == 16 ? SCHED_E_MAX_16 : SCHED_E_MAX))
-        g.sched = nullptr;   // a single K-group per tile (no room to prefetch across tiles) or more experts than the
-                             // schedule table in LDS holds: one tile per workgroup
+    // a single K-group per tile (no room to prefetch across tiles; the 288-row tile fetches the next tile's sorted ids
+    // in its second K-group and needs three) or more experts than the schedule table in LDS holds (the 288-row tile
+    // reads the schedule from global memory): one tile per workgroup
+    if(block_m == 288 ? g.K < 1536 : (g.K < 1024 || g.E > (block_m == 16 ? SCHED_E_MAX_16 : SCHED_E_MAX)))
+        g.sched = nullptr;
     if(g.sched)
     {
         // persistent: as many workgroups per CU as fit (four of the 16-row tile: 4 x 40 KB of LDS, 128 registers; three of
@@ -506,7 +555,10 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
     // of a row block: nearly every expert then has one block, each weight tile one reader, and lines that are
     // dropped first leave the L2 to the activations.  With several blocks per expert the readers of a tile find
     // each other's lines in the L2 and the marking would throw that away.
-    const bool nt = (int64_t)g.T * g.topk * 4 <= (int64_t)g.E * block_m * 3;
+    // (The 288-row tile is chosen for up to 260 rows per expert on average, when all but a few experts in a hundred
+    // still have a single block: up to 15/16 of the block.)
+    const bool nt = block_m == 288 ? (int64_t)g.T * g.topk * 16 <= (int64_t)g.E * block_m * 15
+                                   : (int64_t)g.T * g.topk * 4 <= (int64_t)g.E * block_m * 3;
     // ACT (0 SiLU * up, 1 clamped SwiGLU) only exists for the gate_up stage
 #define GEMM_LAUNCH(MTV, ACTV, NTV) \
     hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, ACTV, NTV>), grid, block, 0, stream, g)
@@ -546,8 +598,8 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
         }
     switch(block_m)
     {
-        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(256, 16)
-    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256}", block_m); return PYHIP_ERR_INVALID;
+        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(256, 16) GEMM_CASE(288, 18)
+    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256,288}", block_m); return PYHIP_ERR_INVALID;
     }
 #undef GEMM_CASE
 #undef GEMM_LAUNCH
@@ -561,8 +613,8 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 {
     PYHIP_REQUIRE(a_q && a_s && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
     PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
-    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256,
-                  "%s: block_m=%d not in {16,32,64,128,256}", name, block_m);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256 || block_m == 288,
+                  "%s: block_m=%d not in {16,32,64,128,256,288}", name, block_m);
     PYHIP_REQUIRE(n_blk >= 0 && n_blk < (1 << 24), "%s: n_blk=%lld", name, (long long)n_blk);
     PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < 0xFFFF0000ll,
                   "%s: activation matrix of %lld rows x %d exceeds the 4 GiB buffer range", name, (long long)a_rows, K);

@@ -163,8 +163,8 @@ def test_sampled_experts_and_properties(layer, T, method):
 
 TILE_CASES = {
     # the token count at which the experts' row counts straddle a tile height: second blocks that are almost empty
-    "dsv3": (8192, (64, 128, 256)), "qwen3": (8192, (64, 128, 256)), "mixtral": (4096, (128, 256)),
-    "gptoss": (4096, (32, 128, 256)),
+    "dsv3": (8192, (64, 128, 256, 288)), "qwen3": (8192, (64, 128, 256, 288)), "mixtral": (4096, (128, 256, 288)),
+    "gptoss": (4096, (32, 128, 256, 288)),
 }
 
 

@@ -86,16 +86,19 @@ def test_row_block_heuristic():
     assert pick_block_m(1024, 8, 256) == 64          # 32
     assert pick_block_m(1056, 8, 256) == 128         # 33
     assert pick_block_m(2048, 8, 256) == 128         # 64
-    assert pick_block_m(8192, 8, 256) == 128         # 256: the largest default tile
+    assert pick_block_m(8192, 8, 256) == 128         # 256 rows per expert, short K loop: 128-row tiles
     # the bf16-activation kernels: twice the mean, at most 64 rows
     assert pick_block_m(128, 8, 256, 7168, True) == 16 and pick_block_m(256, 8, 256, 7168, True) == 16
     assert pick_block_m(512, 8, 256, 7168, True) == 32 and pick_block_m(8192, 8, 256, 7168, True) == 64
     # few experts: the smallest tile that holds twice the mean
     assert pick_block_m(1, 2, 8) == 16 and pick_block_m(32, 2, 8) == 16 and pick_block_m(64, 2, 8) == 32
     assert pick_block_m(128, 2, 8) == 64 and pick_block_m(4096, 2, 8) == 128
-    # the 256-row tile: 120..192 rows per expert and a long K loop
+    # the 256-row tile: 120..224 rows per expert and a long K loop; the 288-row tile: up to 276
     assert pick_block_m(4096, 8, 256, 7168) == 256 and pick_block_m(6144, 8, 256, 7168) == 256
-    assert pick_block_m(3584, 8, 256, 7168) == 128 and pick_block_m(7168, 8, 256, 7168) == 128
+    assert pick_block_m(3584, 8, 256, 7168) == 128 and pick_block_m(7168, 8, 256, 7168) == 256
+    assert pick_block_m(7680, 8, 256, 7168) == 288 and pick_block_m(8192, 8, 256, 7168) == 288
+    assert pick_block_m(8832, 8, 256, 7168) == 288 and pick_block_m(8864, 8, 256, 7168) == 128
+    assert pick_block_m(8192, 8, 256, 7168, True) == 64
     assert pick_block_m(4096, 4, 128, 3072) == 128 and pick_block_m(2048, 8, 128, 4096) == 128
 
 
