@@ -132,7 +132,7 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
  *                tests/contrib/moe/test_moe.py:732-744.  Needs inter % 512 == 0.  At least one of a2 and
  *                a2_q must be given.
  * block_m must equal the block_size the sort ran with and `experts` the expert count it ran with;
- * block_m is 16, 32, 64, 128, 256 or 288; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
+ * block_m is 16, 32, 64, 128, 160, 192, 256 or 288; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
  * workgroup per tile and worst-case block is launched, as the reference does). */
 int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
@@ -237,7 +237,7 @@ int pyhip_moe_zero_fill(void* p, int64_t bytes, pyhip_stream_t stream);
  *   w1, w2, scales, biases, expert_mask, num_local_tokens: as for the step-by-step entry points above
  *   out           bf16 (or fp32 when out_is_f32 != 0) [tokens, hidden]
  *   experts       the expert count the router saw (the length of expert_mask when one is given)
- *   block_m       the row block: 16/32/64, with MXFP4 activations also 128/256/288
+ *   block_m       the row block: 16/32/64, with MXFP4 activations also 128/160/192/256/288
  *   w4a16         0 = MXFP4 activations (pyhip_moe_gemm*_mxfp4), 1 = bf16 activations (pyhip_moe_gemm*_w4a16)
  * pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 give the choices the reference's operator makes inside fused_moe
  * (block_size_M=None, method="auto": src/contrib/fused_moe.py:128-155) as this library makes them (the row block for

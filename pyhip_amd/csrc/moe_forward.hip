@@ -112,15 +112,26 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
     if(w4a16)
         return 64;
     // Prefill sizes: 128 rows, except where a taller tile lets nearly every expert fit ONE row block, so that each weight
-    // tile is read once instead of two or three times.  The 256- and 288-row tiles run one wave per SIMD and have a long
+    // tile is read once instead of two or three times.  The tiles above 128 rows run one wave per SIMD and have a long
     // epilogue, which only pays with a long K loop (hidden >= 6144); the gpt-oss, Qwen3 and Mixtral shapes (hidden 3072 /
-    // 4096) lose 4-13 % with them at the same rows per expert.  DeepSeek-V3 shape, whole layer, ms, tiles of 128 / 256 /
-    // 288 rows: 208 rows per expert 1.94 / 1.85 / 1.87; 224: 2.07 / 1.93 / 1.93; 240: 2.09 / 2.05 / 1.97; 256 (8192 tokens):
-    // 2.29 / 2.69 / 2.06; 264: 2.44 / 3.05 / 2.11; 272: 2.49 / 3.31 / 2.39; 288: 2.57 / 3.53 / 2.97.
-    if(hidden >= 6144 && est >= 120 && est <= 224)
-        return 256;
-    if(hidden >= 6144 && est > 224 && est <= 276)
-        return 288;
+    // 4096) lose 1-13 % with them at the same rows per expert.  DeepSeek-V3 shape, whole layer, ms, tiles of 128 / 160 /
+    // 192 / 256 / 288 rows by expected rows per expert (between machines the order of close neighbours can flip):
+    //    96: 1.28 / 1.33 / 1.36 / 1.50 /  -       160: 2.26 / 1.93 / 1.49 / 1.60 / 1.73      232: 1.97 /  -   /  -   / 1.86 / 1.92
+    //   104: 1.36 / 1.35 / 1.38 / 1.52 / 1.66     168: 2.08 / 2.22 / 1.55 / 1.62 / 1.75      240: 2.09 /  -   /  -   / 1.96 / 1.94
+    //   120: 1.50 / 1.37 / 1.40 / 1.51 / 1.63     176: 2.04 / 2.63 / 1.65 / 1.64 / 1.77      256: 2.26 /  -   /  -   / 2.64 / 2.02
+    //   128: 1.72 / 1.39 / 1.42 / 1.53 / 1.65     192: 1.92 / 2.67 / 2.20 / 1.68 / 1.81      272: 2.46 /  -   /  -   / 3.29 / 2.36
+    //   136: 1.92 / 1.43 / 1.43 / 1.54 / 1.67     208: 1.91 /  -   /  -   / 1.72 / 1.85      288: 2.57 /  -   /  -   / 3.53 / 2.97
+    if(hidden >= 6144)
+    {
+        if(est >= 100 && est <= 132)
+            return 160;
+        if(est > 132 && est <= 172)
+            return 192;
+        if(est > 172 && est <= 236)
+            return 256;
+        if(est > 236 && est <= 276)
+            return 288;
+    }
     return 128;
 }
 
@@ -165,8 +176,8 @@ static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, cons
                   "moe_forward: null pointer");
     PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0 && hidden > 0 && inter > 0, "moe_forward: bad sizes");
     PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 ||
-                      ((block_m == 128 || block_m == 256 || block_m == 288) && !w4a16),
-                  "moe_forward: block_m=%d (16/32/64, and 128/256/288 with MXFP4 activations)", block_m);
+                      ((block_m == 128 || block_m == 160 || block_m == 192 || block_m == 256 || block_m == 288) && !w4a16),
+                  "moe_forward: block_m=%d (16/32/64, and 128/160/192/256/288 with MXFP4 activations)", block_m);
     PYHIP_REQUIRE(!w4a16 || hidden_row_stride == hidden, "moe_forward: the bf16-activation kernels need contiguous rows");
     const Layout l = make_layout(tokens, topk, experts, hidden, inter, block_m, w4a16);
     PYHIP_REQUIRE(workspace && workspace_bytes >= l.total && ((uintptr_t)workspace % 256) == 0,

@@ -48,6 +48,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // The accumulators live in the accumulation registers a0 .. a[16*MT-1], named by hand in the instruction text
     // (mfma_row_group); the clobber reserves that range for the kernel.
     if constexpr(MT >= 16) asm volatile("" ::: "a0", "a255");
+    if constexpr(MT == 12) asm volatile("" ::: "a0", "a191");
+    if constexpr(MT == 10) asm volatile("" ::: "a0", "a159");
     if constexpr(MT == 8) asm volatile("" ::: "a0", "a127");
     if constexpr(MT == 4) asm volatile("" ::: "a0", "a63");
     if constexpr(MT == 2) asm volatile("" ::: "a0", "a31");
@@ -555,10 +557,10 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
     // of a row block: nearly every expert then has one block, each weight tile one reader, and lines that are
     // dropped first leave the L2 to the activations.  With several blocks per expert the readers of a tile find
     // each other's lines in the L2 and the marking would throw that away.
-    // (The 288-row tile is chosen for up to 260 rows per expert on average, when all but a few experts in a hundred
-    // still have a single block: up to 15/16 of the block.)
-    const bool nt = block_m == 288 ? (int64_t)g.T * g.topk * 16 <= (int64_t)g.E * block_m * 15
-                                   : (int64_t)g.T * g.topk * 4 <= (int64_t)g.E * block_m * 3;
+    // (The tiles above 128 rows are chosen so that all but a few experts in a hundred have a single block, up to an
+    // average of 0.8-0.96 of the block: for them the mark stays on up to 15/16 of the block.)
+    const bool nt = block_m > 128 ? (int64_t)g.T * g.topk * 16 <= (int64_t)g.E * block_m * 15
+                                  : (int64_t)g.T * g.topk * 4 <= (int64_t)g.E * block_m * 3;
     // ACT (0 SiLU * up, 1 clamped SwiGLU) only exists for the gate_up stage
 #define GEMM_LAUNCH(MTV, ACTV, NTV) \
     hipLaunchKernelGGL((moe_gemm_mxfp4_kernel<STAGE, MTV, ACTV, NTV>), grid, block, 0, stream, g)
@@ -598,8 +600,9 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
         }
     switch(block_m)
     {
-        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(256, 16) GEMM_CASE(288, 18)
-    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,256,288}", block_m); return PYHIP_ERR_INVALID;
+        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(160, 10) GEMM_CASE(192, 12)
+        GEMM_CASE(256, 16) GEMM_CASE(288, 18)
+    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,160,192,256,288}", block_m); return PYHIP_ERR_INVALID;
     }
 #undef GEMM_CASE
 #undef GEMM_LAUNCH
@@ -613,8 +616,9 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 {
     PYHIP_REQUIRE(a_q && a_s && w && w_s && sorted_ids && sorted_e && num_valid && out, "%s: null pointer", name);
     PYHIP_REQUIRE(K > 0 && K % 512 == 0, "%s: K=%d must be a positive multiple of 512", name, K);
-    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256 || block_m == 288,
-                  "%s: block_m=%d not in {16,32,64,128,256,288}", name, block_m);
+    PYHIP_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 160 || block_m == 192 ||
+                      block_m == 256 || block_m == 288,
+                  "%s: block_m=%d not in {16,32,64,128,160,192,256,288}", name, block_m);
     PYHIP_REQUIRE(n_blk >= 0 && n_blk < (1 << 24), "%s: n_blk=%lld", name, (long long)n_blk);
     PYHIP_REQUIRE(a_rows > 0 && a_rows * (int64_t)(K / 2) < 0xFFFF0000ll,
                   "%s: activation matrix of %lld rows x %d exceeds the 4 GiB buffer range", name, (long long)a_rows, K);

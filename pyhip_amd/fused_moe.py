@@ -75,12 +75,12 @@ def pick_block_m(tokens, topk, experts, hidden=0, w4a16=False):
     sizes so that routers with uneven expert loads do not pay for it: that costs 1-2 % under an even router and saves
     11-17 % under a Zipf(1.1) one (the numbers are quoted beside ``pyhip_moe_pick_block_m``).
 
-    The 256- and 288-row tiles (one wave per SIMD, slower per FLOP) are taken where they save whole passes over the
-    weights: between 120 and 224 expected rows per expert a 128-row tile needs two blocks for most experts and the
-    256-row tile one, between 224 and 276 three against one 288-row block, read with non-temporal loads.  Their long
-    epilogue only pays with a long K loop: DS-V3 (hidden 7168) T = 4096 / 6144: 1.55 / 1.72 ms against 1.69 / 1.92 ms with
-    128 rows, T = 8192: 2.06 ms with 288 rows against 2.29; the gpt-oss, Qwen3 and Mixtral shapes (hidden 3072 / 4096) lose
-    4-13 % with them at the same rows per expert."""
+    The tiles of 160, 192, 256 and 288 rows (one wave per SIMD, slower per FLOP) are taken where they save whole passes
+    over the weights: where a 128-row tile needs two or three blocks for most experts and the taller tile one, read with
+    non-temporal loads (100-132 expected rows per expert: 160 rows; up to 172: 192; up to 236: 256; up to 276: 288).
+    Their long epilogue only pays with a long K loop: DS-V3 (hidden 7168) T = 4096 / 6144: 1.39 / 1.68 ms against
+    1.72 / 1.92 ms with 128 rows, T = 8192: 2.02-2.06 ms with 288 rows against 2.26-2.29; the gpt-oss, Qwen3 and Mixtral shapes
+    (hidden 3072 / 4096) lose 1-13 % with them at the same rows per expert."""
     return int(_lib.load().pyhip_moe_pick_block_m(tokens, topk, experts, hidden, 1 if w4a16 else 0))
 
 

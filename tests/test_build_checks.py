@@ -35,7 +35,7 @@ def _device_asm(tmp_path_factory, src, kernel_re):
 def four_wave_asm(tmp_path_factory):
     """the device assembly of the four-wave GEMM source, compiled once with the library's own flags"""
     text, kernels = _device_asm(tmp_path_factory, SRC, KERNEL_RE)
-    assert len(kernels) == 40, ("expected (gate_up x two activations + down) x six tile heights x two load policies, "
+    assert len(kernels) == 52, ("expected (gate_up x two activations + down) x eight tile heights x two load policies, "
                                 "plus the down GEMM with the atomic epilogue at two tile heights x two load policies")
     return text, kernels
 

@@ -192,12 +192,12 @@ def test_tile_heights_agree_bit_for_bit(layer):
 
 
 @pytest.mark.parametrize("layer", ["dsv3"], indirect=True)
-@pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 256))])
+@pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 160, 192, 256)), (5120, (128, 192, 288))])
 def test_load_policies_agree_bit_for_bit(layer, T, bms):
     """The launch marks the weight loads non-temporal while the rows per expert stay under three quarters of a row
     block (DeepSeek-V3 shape, T=1024: 32 rows per expert, so the 64-, 128- and 256-row tiles take that instance and
-    the 16- and 32-row tiles the other; T=4096: 128 rows per expert, only the 256-row tile does).  A cache policy
-    must not change a bit of the result."""
+    the 16- and 32-row tiles the other; T=4096 and 5120: 128 and 160 rows per expert, the tiles above 128 rows do, up to
+    15/16 of their height).  A cache policy must not change a bit of the result."""
     W = layer
     from pyhip_amd import workloads
     hidden, tw, ti = workloads.make_inputs("dsv3", T)

@@ -138,6 +138,7 @@ def _end_to_end(got32, ref, ref_given_a2, nflip1):
     # 288-row tile: 72 accumulator tiles (8 of them in ordinary registers), ids ring of two, schedule read from global
     # memory; "odd" has three K-groups in gate_up (persistent) and two in down (one workgroup per tile)
     ("mixtral_s", 700, 288, False), ("odd", 640, 288, True), ("longk_s", 330, 288, True), ("tiny", 300, 288, True),
+    ("mixtral_s", 700, 160, False), ("odd", 640, 192, True), ("longk_s", 330, 160, True),
     ("mixtral_s", 33, 32, False),
     ("qwen3_s", 64, 16, False),
     ("qwen3_s", 257, 64, False),

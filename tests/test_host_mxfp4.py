@@ -93,9 +93,11 @@ def test_row_block_heuristic():
     # few experts: the smallest tile that holds twice the mean
     assert pick_block_m(1, 2, 8) == 16 and pick_block_m(32, 2, 8) == 16 and pick_block_m(64, 2, 8) == 32
     assert pick_block_m(128, 2, 8) == 64 and pick_block_m(4096, 2, 8) == 128
-    # the 256-row tile: 120..224 rows per expert and a long K loop; the 288-row tile: up to 276
-    assert pick_block_m(4096, 8, 256, 7168) == 256 and pick_block_m(6144, 8, 256, 7168) == 256
-    assert pick_block_m(3584, 8, 256, 7168) == 128 and pick_block_m(7168, 8, 256, 7168) == 256
+    # long K loop: one row block per expert where a tile of 160 / 192 / 256 / 288 rows holds it
+    assert pick_block_m(3072, 8, 256, 7168) == 128 and pick_block_m(3200, 8, 256, 7168) == 160
+    assert pick_block_m(4096, 8, 256, 7168) == 160 and pick_block_m(4352, 8, 256, 7168) == 192
+    assert pick_block_m(5440, 8, 256, 7168) == 192 and pick_block_m(5632, 8, 256, 7168) == 256
+    assert pick_block_m(6144, 8, 256, 7168) == 256 and pick_block_m(7424, 8, 256, 7168) == 256
     assert pick_block_m(7680, 8, 256, 7168) == 288 and pick_block_m(8192, 8, 256, 7168) == 288
     assert pick_block_m(8832, 8, 256, 7168) == 288 and pick_block_m(8864, 8, 256, 7168) == 128
     assert pick_block_m(8192, 8, 256, 7168, True) == 64
