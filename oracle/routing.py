@@ -8,7 +8,7 @@ The reference has no router on this path: its tests draw ids with ``torch.topk(r
 sum of each group's two best scores, top-8 experts inside them, renormalise).
 
 Pins: invariants (k distinct experts per token, weights sum to 1, at most ``topk_group``
-groups per token) and brute force on tiny inputs (tests/test_oracle_routing.py).
+groups per token) and brute force on tiny inputs (tests/test_oracle_moe.py).
 """
 import numpy as np
 

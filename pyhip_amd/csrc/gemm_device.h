@@ -28,8 +28,7 @@ struct GemmArgs
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
 };
 
-// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales, four at a time: the
-// four MFMAs of one activation row group (16 rows) against the wave's four weight row groups, one assembly statement.
+// acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales.
 // The accumulators are the accumulation registers a[(j*MT + mt)*4 .. +3] of (weight row group j, row group mt), named
 // in the instruction text: the compiler never sees them as values.  (Declared as ordinary vectors, in either register
 // file, about a third of them get renamed on every K-step, get shuffled between the files around the loop and spill.)
@@ -46,38 +45,87 @@ struct GemmArgs
 #define ACC_SPILL_MT0 10
 template <int MT, int MTI>
 constexpr bool acc_in_vgprs() { return (3 * MT + MTI) * 4 >= 256; }
+// One MFMA of a row group: weight row group J (0..3) of the wave against activation row group MTI, K-step U of the
+// K-group.  The four MFMAs of a row group are separate statements so that the kernel can put its other instructions
+// (LDS reads, vector-memory issue) into the gaps between them: an MFMA occupies the matrix pipeline for 16 cycles but
+// the wave's issue port only for four, and instructions issued in those gaps are free, while the same instructions
+// placed after four back-to-back MFMAs delay the next row group (measured on a stream of MFMAs with eight s_nop per
+// row group: + 12 % behind the fourth MFMA, nothing between them).
+template <int U, int MTI, int MT, int J>
+__device__ __forceinline__ void mfma_one(v4i w, v4i a, int ws, int a_scale, v4f* xacc = nullptr)
+{
+    constexpr int A0 = (J * MT + MTI) * 4;
+    static_assert(J == 3 || A0 + 3 < 256, "only weight row group 3 may overflow the accumulation registers");
+    constexpr int WB = (U & 1) * 2 + (J & 1);       // weight-scale byte: (kt%2)*2 + (row%32)/16
+    if constexpr(acc_in_vgprs<MT, MTI>() && J == 3)
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %[xa], %[w], %[a], %[xa], %[ws], %[as] op_sel:[%[wl],%[al],0] "
+                     "op_sel_hi:[%[wh],%[ah],0] cbsz:4 blgp:4"
+                     : [xa] "+v"(*xacc)
+                     : [w] "v"(w), [a] "v"(a), [ws] "v"(ws), [as] "v"(a_scale), [wl] "n"(WB & 1), [wh] "n"(WB >> 1),
+                       [al] "n"(U & 1), [ah] "n"(U >> 1));
+    else
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[%[c]:%[e]], %[w], %[a], a[%[c]:%[e]], %[ws], %[as] "
+                     "op_sel:[%[wl],%[al],0] op_sel_hi:[%[wh],%[ah],0] cbsz:4 blgp:4"
+                     :
+                     : [c] "n"(A0), [e] "n"(A0 + 3), [w] "v"(w), [a] "v"(a), [ws] "v"(ws), [as] "v"(a_scale),
+                       [wl] "n"(WB & 1), [wh] "n"(WB >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
+}
+// the four MFMAs of a row group back to back (the eight-wave kernel, whose two waves per SIMD fill each other's gaps)
 template <int U, int MTI, int MT>
 __device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale,
                                                v4f* xacc = nullptr)
 {
-    constexpr int A0 = (0 * MT + MTI) * 4, A1 = (1 * MT + MTI) * 4, A2 = (2 * MT + MTI) * 4, A3 = (3 * MT + MTI) * 4;
-    static_assert(A2 + 3 < 256, "only weight row group 3 may overflow the accumulation registers");
-    constexpr int W0 = (U & 1) * 2 + 0, W1 = (U & 1) * 2 + 1;       // weight-scale byte: (kt%2)*2 + (row%32)/16
-#define MFMA_TEXT(ACC, ACCE, W, WS, WL, WH)                                                                            \
-    "v_mfma_scale_f32_16x16x128_f8f6f4 a[%[" #ACC "]:%[" #ACCE "]], %[" #W "], %[a], a[%[" #ACC "]:%[" #ACCE "]], %[" #WS  \
-    "], %[as] op_sel:[%[" #WL "],%[al],0] op_sel_hi:[%[" #WH "],%[ah],0] cbsz:4 blgp:4\n\t"
-    if constexpr(acc_in_vgprs<MT, MTI>())
-    {
-        asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
-                     MFMA_TEXT(c2, e2, w2, s23, x0l, x0h)
-                     "v_mfma_scale_f32_16x16x128_f8f6f4 %[xa], %[w3], %[a], %[xa], %[s23], %[as] op_sel:[%[x1l],%[al],0] "
-                     "op_sel_hi:[%[x1h],%[ah],0] cbsz:4 blgp:4\n\t"
-                     : [xa] "+v"(*xacc)
-                     : [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3), [c2] "n"(A2), [e2] "n"(A2 + 3),
-                       [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
-                       [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [x0l] "n"(W0 & 1), [x0h] "n"(W0 >> 1),
-                       [x1l] "n"(W1 & 1), [x1h] "n"(W1 >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
-    }
-    else
-    asm volatile(MFMA_TEXT(c0, e0, w0, s01, x0l, x0h) MFMA_TEXT(c1, e1, w1, s01, x1l, x1h)
-                 MFMA_TEXT(c2, e2, w2, s23, x0l, x0h) MFMA_TEXT(c3, e3, w3, s23, x1l, x1h)
-                 :
-                 : [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3), [c2] "n"(A2), [e2] "n"(A2 + 3),
-                   [c3] "n"(A3), [e3] "n"(A3 + 3), [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
-                   [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [x0l] "n"(W0 & 1), [x0h] "n"(W0 >> 1),
-                   [x1l] "n"(W1 & 1), [x1h] "n"(W1 >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
-#undef MFMA_TEXT
+    mfma_one<U, MTI, MT, 0>(w0, a, ws01, a_scale);
+    mfma_one<U, MTI, MT, 1>(w1, a, ws01, a_scale);
+    mfma_one<U, MTI, MT, 2>(w2, a, ws23, a_scale);
+    mfma_one<U, MTI, MT, 3>(w3, a, ws23, a_scale, xacc);
 }
+
+// ---- Vector-memory issue schedule of one K-group of the four-wave kernel (moe_gemm_mxfp4.hip).
+// A K-group is 4 K-steps x MA row groups; a row group is four MFMAs with a gap after each.  Per wave and K-group the
+// kernel issues NPF prefetch operations (sorted ids, activation DMA, scales) and 16 weight tiles.  They are spread
+// evenly instead of bunched: the texture-address path takes 16 clocks per 1 KB operation and CU, and a wave that finds
+// its queue full stalls at the issue, MFMAs included.
+//   prefetch operation k : gap pslot(k) % 3 of row group pslot(k) / 3, pslot(k) = k * NSLOT / NPF, NSLOT = 9 * MA
+//                          (the gaps 0..2 of the row groups of K-steps 0..2; K-step 3 leaves them time to land)
+//   weight tile (u, j)   : the registers are free once K-step u's MFMAs are issued: u < 3: gap 3 of row group
+//                          (u + 1) * MA + j * MA / 4; u = 3: after the last row group
+// The issue order is the same in every K-group (and in the prologue), which makes "all but the N youngest operations
+// have completed" exact: the functions below count N for the waits.
+template <int MA, int NPF>
+struct VmSchedule
+{
+    static constexpr int NSLOT = 9 * MA;
+    static constexpr int TOTAL = NPF + 16;
+    static constexpr int p_before_slot(int s)      // prefetch operations in slots < s
+    {
+        const int c = (s * NPF + NSLOT - 1) / NSLOT;
+        return s >= NSLOT ? NPF : c < NPF ? c : NPF;
+    }
+    static constexpr int w_rg(int u, int j) { return (u + 1) * MA + j * MA / 4; }
+    static constexpr int w_before_rg(int n)        // weight tiles (u < 3) issued in row groups < n
+    {
+        int c = 0;
+        for(int u = 0; u < 3; u++)
+            for(int j = 0; j < 4; j++)
+                c += w_rg(u, j) < n;
+        return c;
+    }
+    static constexpr int before_rg(int n) { return p_before_slot(3 * n < NSLOT ? 3 * n : NSLOT) + w_before_rg(n); }
+    static constexpr int w_index(int u, int j)
+    {
+        if(u == 3)
+            return NPF + 12 + j;
+        const int n = w_rg(u, j);
+        return p_before_slot(3 * (n + 1) < NSLOT ? 3 * (n + 1) : NSLOT) + 4 * u + j;
+    }
+    // operations younger than the tiles of K-step u (issued one K-group ago) when K-step u starts
+    static constexpr int younger(int u) { return TOTAL - 1 - w_index(u, 3) + before_rg(u * MA); }
+    // operations younger than the last prefetch operation at the end of the K-group
+    // (the weight tiles in gap 3 of its own row group come after it)
+    static constexpr int younger_end() { return 16 - w_before_rg(((NPF - 1) * NSLOT / NPF) / 3); }
+};
+
 template <int R>
 __device__ __forceinline__ float acc_fixed_read()
 {

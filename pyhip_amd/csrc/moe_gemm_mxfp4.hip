@@ -65,12 +65,12 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     constexpr int MR    = TALL ? 2 : 3;        // tiles in the ring of sorted ids / routing weights
     constexpr int NID   = (BM + 63) / 64;     // DMA ops that bring one tile's sorted ids (same for weights)
     constexpr int MPAD  = NID * 64;           // words per meta array
-    constexpr int NM    = (2 * NID + 3) / 4;  // meta DMA ops per wave and K-group (same count in every wave)
-    // VMEM operations per wave and K-group, in issue order: NPF prefetch operations (NM meta, 5*NA activation,
-    // 4 weight-scale) spread between the MFMAs of K-step 0, and 4 weight tiles after each of the 4 K-steps.
-    // A weight tile loaded after K-step u is consumed by K-step u of the next K-group; younger than it at
-    // that point are the tiles of the later K-steps, and for u > 0 this K-group's prefetches and tiles.
-    constexpr int NPF = NM + 5 * NA + 4;
+    constexpr int NM    = (2 * NID + 3) / 4;  // DMA ops per wave that bring a tile's sorted ids and routing weights
+    // VMEM operations per wave and K-group: NPF prefetch operations (5*NA activation, 4 weight-scale) and 16 weight
+    // tiles, in the fixed order of VmSchedule (gemm_device.h), which is what the hand-counted waits rely on.  The
+    // operations that bring the next tile's sorted ids are issued once per tile, ahead of a K-group's schedule, and are
+    // not counted: an operation the counts do not know of only makes a wait cover more than it must.
+    constexpr int NPF = 5 * NA + 4;
     // one LDS stage = the activation tile of a whole K-group (4 K-steps of 128) + its scales
     __shared__ __attribute__((aligned(16))) uint8_t lds_a0[4 * SLOTS * 1024];
     __shared__ __attribute__((aligned(16))) uint8_t lds_a1[4 * SLOTS * 1024];
@@ -81,6 +81,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     constexpr int SCHED_E = TALL ? 0 : MT == 1 ? SCHED_E_MAX_16 : SCHED_E_MAX;
     __shared__ u32 lds_pre[SCHED_E + 1];      // the schedule: row blocks before every expert (and their total),
     __shared__ u32 lds_lid[SCHED_E + 1];      //   local id of every expert
+    __shared__ u32 lds_tab[TALL ? 1 : 128];   // the workgroup's next 64 tiles, decoded (the 288-row tile keeps them in registers)
 
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);   // wave-uniform: keeps descriptors and LDS bases scalar
@@ -102,7 +103,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     const u32 qstride     = gridDim.x >> 3;
     u32 q                 = blockIdx.x >> 3;
     u32 q_end             = 0;
-    int ei                = 0;                        // cursor into the expert list (q only grows)
     if(persistent && !TALL)
     {
         for(int i = tid; i <= g.E; i += GEMM_THREADS)
@@ -115,29 +115,54 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     }
     auto uni = [](u32 v) __attribute__((always_inline)) { return (u32)__builtin_amdgcn_readfirstlane((int)v); };
     // the schedule: row blocks before expert i (i = E: their total) and the local id of expert i; from LDS, or (288-row
-    // tile) from global memory through the scalar cache: uniform addresses, a handful of reads per tile
-    // (the constant address space is what makes the compiler pick scalar loads: a vector load would come with a wait on
-    // the vector-memory counter, which in this pipeline means waiting for every prefetch in flight)
-    typedef const __attribute__((address_space(4))) u32* sched_ptr;
-    auto sched_pre = [&](int i) __attribute__((always_inline)) -> u32 {
-        if constexpr(TALL)
-            return ((sched_ptr)(unsigned long long)g.sched)[i];
-        else
-            return uni(lds_pre[i]);
-    };
-    auto sched_lid = [&](int i) __attribute__((always_inline)) -> u32 {
-        if constexpr(TALL)
-            return ((sched_ptr)(unsigned long long)g.sched)[g.E + 1 + i];
-        else
-            return uni(lds_lid[i]);
-    };
+    // tile, which has no LDS to spare) from global memory
+    auto sched_pre = [&](int i) __attribute__((always_inline)) -> u32 { return TALL ? g.sched[i] : lds_pre[i]; };
+    auto sched_lid = [&](int i) __attribute__((always_inline)) -> u32 { return TALL ? g.sched[g.E + 1 + i] : lds_lid[i]; };
     auto uni4 = [](v4i v) __attribute__((always_inline)) {
         return (v4i){__builtin_amdgcn_readfirstlane(v.x), __builtin_amdgcn_readfirstlane(v.y),
                      __builtin_amdgcn_readfirstlane(v.z), __builtin_amdgcn_readfirstlane(v.w)};
     };
+    // The workgroup's first 64 tiles are decoded before the pipeline starts, one per lane (a binary search over the block
+    // prefixes and a division): stepping to the next tile is then two register (288-row tile: v_readlane) or LDS reads
+    // instead of a dependent chain of schedule reads between two tiles, where nothing else is there to cover them.
+    // (Every wave computes the same table; in LDS they overwrite each other with equal values.  The tiles up to 128 rows
+    // run two workgroups per CU on 128 registers and have none to spare for it.  Tiles beyond the 64th, which only very
+    // large calls have, are decoded one at a time with uniform reads of the schedule.)
+    u32 tab_blk = 0xFFFFFFFFu, tab_nte = 0;       // lane i: row block and weight tile | expert << 16
+    int tab_i   = 0;                              // next entry; 64: the table is used up
+    int ei      = -1;                             // beyond the table: cursor into the expert list (q only grows)
+    auto build_table = [&]() __attribute__((always_inline)) {
+        const u32 qi = q + (u32)lane * qstride;
+        tab_blk      = 0xFFFFFFFFu;
+        tab_nte      = 0;
+        if(qi < q_end && qi >= q)                 // (qi >= q: no wrap-around)
+        {
+            int lo = 0, hi = g.E - 1;             // first expert whose tiles end beyond qi
+            while(lo < hi)
+            {
+                const int mid = (lo + hi) >> 1;
+                if(sched_pre(mid + 1) * (u32)g.n_tiles > qi)
+                    hi = mid;
+                else
+                    lo = mid + 1;
+            }
+            const u32 p0    = sched_pre(lo);
+            const u32 nb    = sched_pre(lo + 1) - p0;
+            const u32 local = qi - p0 * (u32)g.n_tiles;
+            const u32 nt    = local / nb;
+            tab_blk         = p0 + (local - nt * nb);
+            tab_nte         = nt | (sched_lid(lo) << 16);
+        }
+        if constexpr(!TALL)
+        {
+            lds_tab[lane]      = tab_blk;
+            lds_tab[64 + lane] = tab_nte;
+            tab_blk = tab_nte = 0;                // (not kept in registers)
+        }
+    };
     if(persistent)
     {
-        const u32 tiles = sched_pre(g.E) * (u32)g.n_tiles;
+        const u32 tiles = uni(sched_pre(g.E)) * (u32)g.n_tiles;
         const u32 chunk = (tiles + 7u) >> 3;
         // (Every workgroup of the launch takes part, also when the last round of an XCD's run is nearly empty.  Letting only
         // as many take part as make the rounds even (113 tiles on 96 workgroups: 57 with two tiles each) was measured and is
@@ -146,19 +171,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         q += (u32)xcd * chunk;
         q_end = (u32)(xcd + 1) * chunk < tiles ? (u32)(xcd + 1) * chunk : tiles;
         if(q < q_end)
-        {
-            // first expert whose tiles end beyond q
-            int lo = 0, hi = g.E - 1;
-            while(lo < hi)
-            {
-                const int mid = (lo + hi) >> 1;
-                if(sched_pre(mid + 1) * (u32)g.n_tiles > q)
-                    hi = mid;
-                else
-                    lo = mid + 1;
-            }
-            ei = lo;
-        }
+            build_table();
     }
     auto decode = [&](TileId& t) __attribute__((always_inline)) {
         t.valid = false;
@@ -166,14 +179,32 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         {
             if(q >= q_end)
                 return;
-            while(q >= sched_pre(ei + 1) * (u32)g.n_tiles)
-                ei++;
-            const u32 p0    = sched_pre(ei);
-            const u32 nb    = sched_pre(ei + 1) - p0;
-            const u32 local = q - p0 * (u32)g.n_tiles;
-            t.nt            = (int)(local / nb);
-            t.m_blk         = (int)(p0 + (local - (u32)t.nt * nb));
-            t.e             = (int)sched_lid(ei);
+            if(tab_i < 64)
+            {
+                const u32 blk = TALL ? (u32)__builtin_amdgcn_readlane((int)tab_blk, tab_i) : uni(lds_tab[tab_i]);
+                const u32 nte = TALL ? (u32)__builtin_amdgcn_readlane((int)tab_nte, tab_i) : uni(lds_tab[64 + tab_i]);
+                tab_i++;
+                t.m_blk = (int)blk;
+                t.nt    = (int)(nte & 0xFFFFu);
+                t.e     = (int)(nte >> 16);
+            }
+            else
+            {
+                auto pre_u = [&](int i) __attribute__((always_inline)) -> u32 {
+                    typedef const __attribute__((address_space(4))) u32* sched_ptr;    // scalar loads
+                    return TALL ? ((sched_ptr)(unsigned long long)g.sched)[i] : uni(lds_pre[i]);
+                };
+                if(ei < 0)
+                    ei = 0;
+                while(q >= pre_u(ei + 1) * (u32)g.n_tiles)
+                    ei++;
+                const u32 p0    = pre_u(ei);
+                const u32 nb    = pre_u(ei + 1) - p0;
+                const u32 local = q - p0 * (u32)g.n_tiles;
+                t.nt            = (int)(local / nb);
+                t.m_blk         = (int)(p0 + (local - (u32)t.nt * nb));
+                t.e             = (int)(TALL ? pre_u(g.E + 1 + ei) : uni(lds_lid[ei]));
+            }
             q += qstride;
         }
         else
@@ -189,37 +220,22 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         }
         t.valid = true;
     };
-    // sorted ids and routing weights of a tile's rows -> LDS meta buffer `buf` (DMA, 64 rows per op, NM ops per
-    // wave; `on` = false issues the same operations with zero-range descriptors)
-    auto dma_meta = [&](const TileId& t, int buf, bool on) __attribute__((always_inline)) {
-        const v4i rid = make_rsrc(g.sorted_ids + (size_t)t.m_blk * BM, BM * 4);
-        const v4i rwt = make_rsrc(g.sorted_w + (size_t)t.m_blk * BM, BM * 4);
-#pragma unroll
-        for(int i = 0; i < NM; i++)
-        {
-            const int o     = wave + 4 * i;               // op index: [0, NID) ids, [NID, 2*NID) weights, beyond: nothing
-            const bool wts  = o >= NID;
-            const int oo    = wts ? o - NID : o;
-            const bool real = on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
-            // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
-            const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
-            const u32 dst   = uni(real ? lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
-            vm_dma_b32_fresh_sgprs((oo * 64 + lane) * 4, rs, dst);
-        }
-    };
-
     // ---- load side of the pipeline: descriptors and per-lane offsets of the tile being prefetched
     // (every prefetch is issued unconditionally; when there is no tile left to prefetch the descriptors get
     // a zero range, so the hardware drops the accesses and the instruction stream stays the same)
     v4i wrs[2];    // weight rows of this wave: stage 1 [0] gate, [1] up (2 row groups each); stage 2 [0] all 4 groups
     v4i wsrs[2];   // their scale tiles, same split (rows j = 0,1 share a 32-row scale tile, so do j = 2,3)
-    v4i ars, asrs; // activations and their scales
+    // activations and their scales: the same for every tile (rows that fetch nothing carry an out-of-range offset)
+    const v4i ars  = make_rsrc(g.a_q, (u32)((size_t)g.a_rows * Kb));
+    const v4i asrs = make_rsrc(g.a_s, (u32)((size_t)g.a_rows * g.SK));
     int a_off[NA], as_off[NA];        // this lane's byte offsets inside a_q / a_s at K = 0, per DMA slot
     // DMA lane mapping: four consecutive lanes fetch the 64 contiguous bytes of one row and K-step (a gather
     // with one row per lane costs four times the address-pipeline cycles).  LDS therefore holds a (row group,
     // K-step) block row-major, 16 rows x 64 B; the 16 B chunk c of row r sits in slot c ^ ((r / 2) % 4), which makes
     // the operand reads (lane = K-block * 16 + row) conflict-free: measured 4 LDS cycles per ds_read_b128, against
     // 8 for c ^ (r / 4) or for no swizzle at all.
+    // (Eight lanes per row, the 128 B line that a row contributes to a pair of K-steps, was built and measured as well:
+    // the same time, bit-identical, and one more offset register per slot, which the 128-row tile does not have.)
     const int dma_row   = lane >> 2;
     const int dma_chunk = (lane & 3) ^ ((lane >> 3) & 3);
     const int rd_a      = r * 64 + ((kb ^ ((r >> 1) & 3)) * 16);   // operand read offset inside a 1 KB block
@@ -227,8 +243,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     auto setup_null = [&]() __attribute__((always_inline)) {
         wrs[0] = wrs[1] = make_rsrc(g.w, 0);
         wsrs[0] = wsrs[1] = make_rsrc(g.w_s, 0);
-        ars  = make_rsrc(g.a_q, 0);
-        asrs = make_rsrc(g.a_s, 0);
+#pragma unroll
+        for(int i = 0; i < NA; i++)
+            a_off[i] = as_off[i] = (int)0xFFFF0000u;
     };
     // Row groups of a tile that hold at least one real row.  The sort pads every expert's rows at the END of
     // its last block, so the real rows of a block are a prefix.  Padded rows send their activation fetches out
@@ -265,8 +282,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             wrs[0] = wrs[1] = make_rsrc(g.w + row * Kb, (u32)(64 * Kb));
             wsrs[0] = wsrs[1] = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)(2 * sc_tile));
         }
-        ars  = make_rsrc(g.a_q, (u32)((size_t)g.a_rows * Kb));
-        asrs = make_rsrc(g.a_s, (u32)((size_t)g.a_rows * g.SK));
 #pragma unroll
         for(int i = 0; i < NA; i++)
         {
@@ -301,18 +316,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         else
             return normal;
     };
-    auto dma_group = [&](auto S, int ks) __attribute__((always_inline)) {
-        constexpr int s = decltype(S)::value;
-        static_for<NA>([&](auto II) __attribute__((always_inline)) {
-            constexpr int i = decltype(II)::value;
-            static_for<4>([&](auto U) __attribute__((always_inline)) {
-                constexpr int u = decltype(U)::value;
-                constexpr int imm = (u * SLOTS + 4 * i) * 1024;
-                vm_dma_b128<u * 64, imm>(a_off[i], ars, ks * 256, slot_base(II, std::integral_constant<int, imm>{}, lds_a[s]));
-            });
-            vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, ks * 16, slot_base(II, std::integral_constant<int, 4 * i * 256>{}, lds_s[s]));
-        });
-    };
     v4i wf[4][4];
     int w_sc[2][4];
     // per-lane offsets of the wave's row groups inside wrs[] / of its scale dwords inside wsrs[]; the half that
@@ -321,14 +324,6 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1
     const int w_half     = (STAGE == 2) ? 32 * Kb : 0;
     const int ws_half    = (STAGE == 2) ? (g.SC / 8) * 256 : 0;
-    auto load_wscales = [&](auto S, int ks) __attribute__((always_inline)) {
-        constexpr int s = decltype(S)::value;
-#pragma unroll
-        for(int h = 0; h < 2; h++)
-#pragma unroll
-            for(int c = 0; c < 2; c++)
-                vm_load_b32<0>(w_sc[s][h * 2 + c], lane * 4 + c * 256, wsrs[h], ks * 512 + h * ws_half);
-    };
     auto load_wtile = [&](auto U, auto J, int kt) __attribute__((always_inline)) {
         constexpr int u = decltype(U)::value, j = decltype(J)::value;
         vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
@@ -345,6 +340,69 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     };
 
     // ---------------------------------------------------------------- pipeline
+    constexpr int MA = MT;                    // row groups that take part in the MFMAs
+    using VS = VmSchedule<MA, NPF>;
+    static_assert(VS::younger(0) <= 63 && VS::younger(1) <= 63 && VS::younger(2) <= 63 && VS::younger(3) <= 63,
+                  "the vector-memory counter has six bits");
+    // sorted ids and routing weights of a tile's rows -> LDS meta buffer `buf` (DMA, 64 rows per operation, spread over
+    // the four waves)
+    auto dma_meta = [&](const TileId& t, int buf) __attribute__((always_inline)) {
+        const v4i rid = make_rsrc(g.sorted_ids + (size_t)t.m_blk * BM, BM * 4);
+        const v4i rwt = make_rsrc(g.sorted_w + (size_t)t.m_blk * BM, BM * 4);
+#pragma unroll
+        for(int i = 0; i < NM; i++)
+        {
+            const int o    = wave + 4 * i;               // op index: [0, NID) ids, [NID, 2*NID) weights, beyond: nothing
+            const bool wts = o >= NID;
+            const int oo   = wts ? o - NID : o;
+            if(o < 2 * NID && (!wts || g.sorted_w != nullptr))
+                vm_dma_b32_fresh_sgprs((oo * 64 + lane) * 4, uni4(wts ? rwt : rid),
+                                       uni(lds_addr_of(&lds_meta[buf][(wts ? MPAD : 0) + oo * 64])));
+        }
+    };
+    // prefetch operation K (0 <= K < NPF) of a K-group: TS = the LDS stage / scale register set it fills, kpre = the
+    // K-group it fetches
+    auto prefetch_op = [&](auto KK, auto TS, int kpre) __attribute__((always_inline)) {
+        constexpr int k = decltype(KK)::value, ts = decltype(TS)::value;
+        if constexpr(k < 5 * NA)
+        {
+            constexpr int i = k / 5, sub = k % 5;
+            using II = std::integral_constant<int, i>;
+            if constexpr(sub < 4)
+            {
+                constexpr int imm = (sub * SLOTS + 4 * i) * 1024;
+                vm_dma_b128<sub * 64, imm>(a_off[i], ars, kpre * 256, slot_base(II{}, std::integral_constant<int, imm>{}, lds_a[ts]));
+            }
+            else
+                vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, kpre * 16, slot_base(II{}, std::integral_constant<int, 4 * i * 256>{}, lds_s[ts]));
+        }
+        else
+        {
+            constexpr int h = (k - 5 * NA) / 2, c = (k - 5 * NA) % 2;
+            vm_load_b32<0>(w_sc[ts][h * 2 + c], lane * 4 + c * 256, wsrs[h], kpre * 512 + h * ws_half);
+        }
+    };
+    // the vector-memory operations of gap G of row group N (see VmSchedule)
+    auto issue_gap = [&](auto N, auto G, auto TS, int kpre) __attribute__((always_inline)) {
+        constexpr int n = decltype(N)::value, gp = decltype(G)::value;
+        if constexpr(gp < 3)
+        {
+            if constexpr(3 * n + gp < VS::NSLOT)
+            {
+                constexpr int k0 = VS::p_before_slot(3 * n + gp), k1 = VS::p_before_slot(3 * n + gp + 1);
+                static_for<k1 - k0>([&](auto Q) __attribute__((always_inline)) {
+                    prefetch_op(std::integral_constant<int, k0 + decltype(Q)::value>{}, TS, kpre);
+                });
+            }
+        }
+        else
+            static_for<12>([&](auto UJ) __attribute__((always_inline)) {
+                constexpr int u = decltype(UJ)::value / 4, j = decltype(UJ)::value % 4;
+                if constexpr(VS::w_rg(u, j) == n)
+                    load_wtile(std::integral_constant<int, u>{}, std::integral_constant<int, j>{}, kpre * 4 + u);
+            });
+    };
+
     TileId cur, nxt;
     decode(cur);
     if(!cur.valid)
@@ -353,13 +411,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     setup_load(cur, g.sorted_ids + (size_t)cur.m_blk * BM);
     int ma     = count_groups(g.sorted_ids + (size_t)cur.m_blk * BM);   // active row groups of the current tile
     int ma_nxt = ma;                                                    // ... and of the next one
-    // prologue, in the K-group's issue order: this tile's ids/weights, activation K-group 0, weight scales of
-    // group 0, weight tiles of K-steps 0..3
-    dma_meta(cur, 0, true);
-    dma_group(std::integral_constant<int, 0>{}, 0);
-    load_wscales(std::integral_constant<int, 0>{}, 0);
-    static_for<4>([&](auto U) __attribute__((always_inline)) { load_wtiles(U, decltype(U)::value); });
-    wait_vmcnt_barrier<16>();         // everything older than the weight tiles has landed
+    // prologue: a K-group's vector-memory operations in the K-group's issue order, without the MFMAs: this tile's
+    // ids / routing weights, activation K-group 0 into stage 0, weight scales and weight tiles of K-steps 0..3
+    dma_meta(cur, 0);
+    static_for<4 * MA>([&](auto N) __attribute__((always_inline)) {
+        static_for<4>([&](auto G) __attribute__((always_inline)) { issue_gap(N, G, std::integral_constant<int, 0>{}, 0); });
+    });
+    load_wtiles(std::integral_constant<int, 3>{}, 3);
+    wait_vmcnt_barrier<VS::younger_end()>();      // everything but the youngest weight tiles has landed
     decode(nxt);                      // (without a schedule there is no next tile)
     zero_acc();
     int ks = 0;
@@ -376,6 +435,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         //     next tile (into the other LDS stage, whose readers left at the last barrier)
         if(last)
         {
+            // (kept a branch: turned into selects, the set-up would run, and cost its scalar chain, in every K-group)
+            asm volatile("" ::: "memory");
             if(nxt.valid)
             {
                 setup_load(nxt, lds_meta[mb_nxt]);
@@ -386,46 +447,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         }
         // (with a ring of two the slot still belongs to the previous tile, whose epilogue a slower wave may not have
         // finished before the barrier that ends this tile's first K-group: the fetch waits for the second K-group)
-        const bool meta_on = ks == (TALL ? 1 : 0) && nxt.valid;
-        const v4i rid = make_rsrc(g.sorted_ids + (size_t)nxt.m_blk * BM, BM * 4);
-        const v4i rwt = make_rsrc(g.sorted_w + (size_t)nxt.m_blk * BM, BM * 4);
-        // prefetch operation K of this K-group (0 <= K < NPF)
-        auto prefetch_op = [&](auto KK) __attribute__((always_inline)) {
-            constexpr int k = decltype(KK)::value;
-            if constexpr(k < NM)
-            {
-                // ids/weights of the NEXT tile into the meta ring (first K-group of a tile only; two tiles ahead
-                // of the slot any wave can still be reading in its epilogue)
-                const int o     = wave + 4 * k;           // op index: [0, NID) ids, [NID, 2*NID) weights, beyond: nothing
-                const bool wts  = o >= NID;
-                const int oo    = wts ? o - NID : o;
-                const bool real = meta_on && o < 2 * NID && (!wts || g.sorted_w != nullptr);
-                // a switched-off operation still writes (zeros) to LDS: point it at the dummy area
-                const v4i rs    = uni4(real ? (wts ? rwt : rid) : make_rsrc(g.sorted_ids, 0));
-                const u32 dst   = uni(real ? lds_addr_of(&lds_meta[mb_nxt][(wts ? MPAD : 0) + oo * 64]) : lds_addr_of(lds_dummy));
-                vm_dma_b32_fresh_sgprs((oo * 64 + lane) * 4, rs, dst);
-            }
-            else if constexpr(k < NM + 5 * NA)
-            {
-                constexpr int i = (k - NM) / 5, sub = (k - NM) % 5;
-                using II = std::integral_constant<int, i>;
-                if constexpr(sub < 4)
-                {
-                    constexpr int imm = (sub * SLOTS + 4 * i) * 1024;
-                    vm_dma_b128<sub * 64, imm>(a_off[i], ars, kpre * 256, slot_base(II{}, std::integral_constant<int, imm>{}, lds_a[p ^ 1]));
-                }
-                else
-                    vm_dma_b32<0, 4 * i * 256>(as_off[i], asrs, kpre * 16, slot_base(II{}, std::integral_constant<int, 4 * i * 256>{}, lds_s[p ^ 1]));
-            }
-            else
-            {
-                constexpr int h = (k - NM - 5 * NA) / 2, c = (k - NM - 5 * NA) % 2;
-                vm_load_b32<0>(w_sc[p ^ 1][h * 2 + c], lane * 4 + c * 256, wsrs[h], kpre * 512 + h * ws_half);
-            }
-        };
-        // MFMAs, prefetches and weight loads of the K-group
-        constexpr int MA  = MT;                   // row groups that take part
-        constexpr int PPM = (NPF + MA - 1) / MA;  // prefetch operations issued after each row group's MFMAs
+        if(ks == (TALL ? 1 : 0) && nxt.valid)
+            dma_meta(nxt, mb_nxt);
+        using TS = std::integral_constant<int, p ^ 1>;
         // The activation operand of a row group and its scale dword (one per 16-row group and K-group, op_sel picks the
         // K-step's byte) are read RA row groups ahead of the MFMAs that consume them, across K-step boundaries, through
         // a ring of RA + 1 register sets: two ahead with two waves per SIMD, four in the one-wave-per-SIMD 256-row
@@ -443,55 +467,42 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         __builtin_amdgcn_sched_barrier(0);
         static_for<4>([&](auto U) __attribute__((always_inline)) {
             constexpr int u = decltype(U)::value;
-            // (3) MFMAs of K-step 4*ks + u, tile operands two reads ahead of their MFMAs.  The weight tiles of
-            //     this K-step (and, at u = 0, the weight scales) were requested one K-group ago.
-            //     Issue order of a K-group: the prefetches during K-step 0; the tiles of K-steps 0, 1, 2 of the
-            //     prefetched K-group one at a time during K-steps 1, 2, 3 (spread over the row groups: four 1 KB loads
-            //     back to back from every wave at once fill the address unit's queue and stall the issuing waves);
-            //     the tiles of K-step 3 after K-step 3.  Younger than the tiles of K-step u when it starts: u = 0: those
-            //     of K-steps 1, 2, 3; u = 1, 2, 3: two more K-steps' tiles and this K-group's prefetches.
-            constexpr int YOUNGER = u == 0 ? 12 : 8 + NPF;
+            // MFMAs of K-step 4*ks + u.  Its weight tiles (and, at u = 0, the weight scales) were requested one K-group
+            // ago; VS::younger counts what has been issued since.
+            constexpr int YOUNGER = VS::younger(u);
             wait_vm_tiles<YOUNGER>(wf[u][0], wf[u][1], wf[u][2], wf[u][3]);
             if(u == 0)
                 wait_vm_scales<YOUNGER>(w_sc[p][0], w_sc[p][1], w_sc[p][2], w_sc[p][3]);
             static_for<MA>([&](auto M) __attribute__((always_inline)) {
                 constexpr int mt = decltype(M)::value;
                 constexpr int n  = u * MA + mt;                // position in the K-group's sequence of row groups
-                if constexpr(n + RA < 4 * MA)
-                    lds_read(std::integral_constant<int, n + RA>{});
+                using N = std::integral_constant<int, n>;
                 const v4i af  = af_r[n % (RA + 1)];
                 const int asc = asc_all[mt];
                 __builtin_amdgcn_sched_barrier(0);
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
-                if constexpr(acc_in_vgprs<MT, mt>())
-                    mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
-                                              w_sc[p][2 + (u >> 1)], asc, &xacc[mt - ACC_SPILL_MT0]);
-                else
-                    mfma_row_group<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][0 + (u >> 1)],
-                                              w_sc[p][2 + (u >> 1)], asc);
-                // K-step 0 carries this K-group's prefetches, a few after each row group's MFMAs, so that their
-                // issue overlaps the matrix pipeline instead of preceding it
-                if constexpr(u == 0)
-                    static_for<PPM>([&](auto Q) __attribute__((always_inline)) {
-                        constexpr int k = mt * PPM + decltype(Q)::value;
-                        if constexpr(k < NPF)
-                            prefetch_op(std::integral_constant<int, k>{});
-                    });
-                // (4) weight tiles of the previous K-step of the prefetched K-group into the registers it consumed
-                if constexpr(u > 0)
-                    static_for<4>([&](auto J) __attribute__((always_inline)) {
-                        if constexpr(mt == (decltype(J)::value * MA) / 4)
-                            load_wtile(std::integral_constant<int, u - 1>{}, J, kpre * 4 + u - 1);
-                    });
-                __builtin_amdgcn_sched_barrier(0);
+                static_for<4>([&](auto J) __attribute__((always_inline)) {
+                    constexpr int j = decltype(J)::value;
+                    v4f* xa = nullptr;
+                    if constexpr(acc_in_vgprs<MT, mt>() && j == 3)
+                        xa = &xacc[mt - ACC_SPILL_MT0];
+                    mfma_one<u, mt, MT, j>(wf[u][j], af, w_sc[p][(j >> 1) * 2 + (u >> 1)], asc, xa);
+                    __builtin_amdgcn_sched_barrier(0);
+                    // the gap after the MFMA: the operand read of the row group RA ahead, then this gap's share of the
+                    // K-group's vector-memory operations
+                    if constexpr(j == 0 && n + RA < 4 * MA)
+                        lds_read(std::integral_constant<int, n + RA>{});
+                    issue_gap(N{}, J, TS{}, kpre);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             });
             __builtin_amdgcn_sched_barrier(0);
             if constexpr(u == 3)
                 load_wtiles(U, kpre * 4 + u);
             __builtin_amdgcn_sched_barrier(0);
         });
-        // (5) the 16 weight loads above are the only VMEM ops younger than this group's DMAs
-        wait_vmcnt_barrier<16>();
+        // the weight tiles issued since the last prefetch operation are the only operations that may still be under way
+        wait_vmcnt_barrier<VS::younger_end()>();
         ks++;
         if(last)
         {

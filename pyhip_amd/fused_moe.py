@@ -42,26 +42,36 @@ def _is_shuffled(w):
     return bool(getattr(w, "is_shuffled", False))
 
 
-_shuffle_cache = {}
+_shuffle_cache = {}          # id(source storage) -> {view key: (tensor version, re-tiled copy)}
+_SHUFFLE_CACHE_STORAGES = 8  # plain-layout weight storages remembered at once (each entry holds a full re-tiled copy)
 
 
 def _shuffled_u8(w):
     """uint8 view of an MXFP4 weight tensor in the pre-shuffled layout the kernels read.  Plain-layout weights
-    ([E, N, K/2] row-major, ``is_shuffled`` unset) are shuffled once and remembered per storage (the reference's
-    kernels take both layouts, src/contrib/fused_moe.py:410,480; here the plain layout costs one re-tiling pass on
-    first use and a second copy of the weights)."""
+    ([E, N, K/2] row-major, ``is_shuffled`` unset) are shuffled once and remembered (the reference's kernels take both
+    layouts, src/contrib/fused_moe.py:410,480; here the plain layout costs one re-tiling pass on first use and a second
+    copy of the weights).  An entry belongs to the source tensor's storage object: it is dropped by a finalizer when that
+    storage is freed, so a new tensor that lands at the same address never finds a stale copy, and an in-place change
+    of the source (its version counter) invalidates it."""
     wu = _as_u8(w)
     if _is_shuffled(w):
         return wu
+    import weakref
     from .mxfp4 import shuffle_weight
-    key = (wu.data_ptr(), tuple(wu.shape), str(wu.device))
-    hit = _shuffle_cache.get(key)
+    storage = wu.untyped_storage()
+    sid = id(storage)            # the storage's Python object lives exactly as long as the storage
+    views = _shuffle_cache.get(sid)
+    if views is None:
+        while len(_shuffle_cache) >= _SHUFFLE_CACHE_STORAGES:
+            _shuffle_cache.pop(next(iter(_shuffle_cache)))      # oldest first
+        views = _shuffle_cache[sid] = {}
+        weakref.finalize(storage, _shuffle_cache.pop, sid, None)
+    key = (wu.storage_offset(), tuple(wu.shape), tuple(wu.stride()))
+    hit = views.get(key)
     if hit is not None and hit[0] == wu._version:
         return hit[1]
-    if len(_shuffle_cache) >= 16:
-        _shuffle_cache.clear()
     out = shuffle_weight(wu.contiguous())
-    _shuffle_cache[key] = (wu._version, out)
+    views[key] = (wu._version, out)
     return out
 
 

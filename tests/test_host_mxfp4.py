@@ -127,3 +127,41 @@ def test_library_makes_the_same_choices():
             for w4 in (0, 1):
                 assert lib.pyhip_moe_pick_block_m(T, k, E, H, w4) == pick_block_m(T, k, E, H, bool(w4)), (T, k, E, H, w4)
             assert bool(lib.pyhip_moe_pick_w4a16(T, k, E, H)) == pick_w4a16(T, k, E, H), (T, k, E, H)
+
+
+def test_plain_layout_cache_follows_the_source_storage():
+    """The operator re-tiles plain-layout weights once and remembers the copy.  The copy must die with the source:
+    a second tensor of the same shape that reuses the freed address (and starts at version 0 like the first) has to
+    be re-tiled from its own bytes."""
+    import gc
+    import importlib
+    fm = importlib.import_module("pyhip_amd.fused_moe")      # (the package re-exports the function under the module's name)
+    fm._shuffle_cache.clear()
+    g = torch.Generator().manual_seed(5)
+    a = torch.randint(0, 256, (2, 64, 128), dtype=torch.uint8, generator=g)
+    ptr = a.data_ptr()
+    sa = fm._shuffled_u8(a)
+    assert (sa == mxfp4.shuffle_weight(a)).all() and len(fm._shuffle_cache) == 1
+    assert fm._shuffled_u8(a) is sa                                  # hit
+    assert fm._shuffled_u8(a.view(torch.int8)) is sa                 # another view of the same storage: hit
+    a[0, 0, 0] ^= 0xFF                                               # in-place change: version moves, copy is redone
+    sa2 = fm._shuffled_u8(a)
+    assert sa2 is not sa and (sa2 == mxfp4.shuffle_weight(a)).all()
+    del a, sa, sa2
+    gc.collect()
+    assert len(fm._shuffle_cache) == 0                               # freed with its source
+    same_address = False
+    for _ in range(8):                                               # the allocator normally hands the block out again
+        b = torch.randint(0, 256, (2, 64, 128), dtype=torch.uint8, generator=g)
+        same_address = same_address or b.data_ptr() == ptr
+        assert (fm._shuffled_u8(b) == mxfp4.shuffle_weight(b)).all()
+        del b
+        gc.collect()
+        assert len(fm._shuffle_cache) == 0
+    # (whether or not the address came back, every result above was made from the tensor's own bytes)
+    # the number of storages remembered at once is bounded
+    keep = [torch.randint(0, 256, (1, 16, 64), dtype=torch.uint8, generator=g) for _ in range(fm._SHUFFLE_CACHE_STORAGES + 3)]
+    for t in keep:
+        fm._shuffled_u8(t)
+    assert len(fm._shuffle_cache) == fm._SHUFFLE_CACHE_STORAGES
+    fm._shuffle_cache.clear()
