@@ -18,6 +18,10 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
                from HIP events recorded on the launch stream around that launch in a separate, untimed pass
                of the step-by-step path; traffic is read from the committed counter summary under profiles/
   cpu_baseline the CPU oracle (oracle/moe.py) on a bounded sample of the headline workload
+
+Measurement modes.  ``--epilogue-comparison``, ``--tile256-comparison TOKENS`` and ``--calibrate-copy MIB`` are not part
+of the default line: each adds one extra object to it (or, for the copy, only extra launches for a counter run) and
+exists so that the command lines quoted in ``profiles/*.txt`` run from this file alone.
 """
 import argparse
 import json
@@ -64,6 +68,8 @@ def parse():
                          "256-row tile and the eight-wave 256-row tile with both operands through LDS")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
+    ap.add_argument("--print-kernel-sources-digest", action="store_true",
+                    help="print the digest that profiles/fused_moe_dsv3_hbm_traffic.txt records next to its counters, and exit")
     return ap.parse_args()
 
 
@@ -231,17 +237,34 @@ def graph_replay_ms(torch, fused_moe, W, res, steps, block_m, method="auto"):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+KERNEL_SOURCES = ("moe_gemm_mxfp4.hip", "gemm_device.h", "common.h", "quant_device.h")
+
+
+def kernel_sources_digest():
+    """sha256 over the sources the measured GEMM kernels are compiled from"""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "pyhip_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(kernel_key):
     """HBM-side bytes per launch of a kernel from the committed counter summary (lines of the form
-    `traffic_bytes_per_launch <key> <bytes>`, written when the counters were collected, with the commit they
-    were collected at); None when the summary has no such line"""
+    `traffic_bytes_per_launch <key> <bytes>`, written when the counters were collected, next to a line
+    `kernel_sources_sha256 <digest>` of the kernel sources they were collected with).  None when the summary has no
+    such line, or when the kernel sources have changed since: a counter reading of other code is not reported."""
     try:
         text = open(TRAFFIC_FILE).read()
     except OSError:
         return None, None
     m = re.search(r"^traffic_bytes_per_launch\s+%s\s+([0-9.eE+]+)" % re.escape(kernel_key), text, re.M)
     c = re.search(r"^collected_at\s+(.+)$", text, re.M)
-    return (float(m.group(1)) if m else None), (c.group(1).strip() if c else None)
+    d = re.search(r"^kernel_sources_sha256\s+([0-9a-f]{64})", text, re.M)
+    if m is None or d is None or d.group(1) != kernel_sources_digest():
+        return None, None
+    return float(m.group(1)), (c.group(1).strip() if c else None)
 
 
 class LazyExperts:
@@ -304,6 +327,9 @@ def point_record(shape, tokens, r):
 
 def main():
     a = parse()
+    if a.print_kernel_sources_digest:
+        print(kernel_sources_digest())
+        return
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU only (--gpus %d requested); expert-parallel sharding over "
               "several GPUs is not built." % a.gpus, file=sys.stderr)

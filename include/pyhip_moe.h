@@ -272,7 +272,10 @@ int pyhip_moe_forward_routed(const void* hidden_bf16, int64_t hidden_row_stride,
  * hipFree, no allocating library routine); calls whose intermediates exceed the capacity are refused with error 1
  * before anything is launched (decode-sized calls fit: DeepSeek-V3 shape, 128 tokens, bf16 activations: 35 MiB).
  * Same arguments, kernels and results as pyhip_moe_forward.  All calls on one GPU share the array: calls that
- * overlap on one GPU (two streams, two threads) race; nothing in the array needs clearing between calls. */
+ * overlap on one GPU (two streams, two threads) race; nothing in the array needs clearing between calls.
+ * pyhip_moe_forward_static_capacity() returns the array's size and makes the runtime map the array on the current
+ * device: callers that capture the layer call in a graph run it once per device beforehand, so that the first call
+ * inside the capture has nothing left to set up. */
 int64_t pyhip_moe_forward_static_capacity(void);
 int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
                              const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,

@@ -29,8 +29,10 @@ def _run(cmd):
 
 
 CO_DIR = os.path.join(HERE, "co")
-# sources whose kernels are also shipped as stand-alone code objects (see build_co)
-CO_SOURCES = ["moe_quant.hip", "moe_reduce.hip", "moe_gemm_mxfp4.hip"]
+# every source that holds kernels is also shipped as a stand-alone code object (see build_co); the rest of SOURCES
+# (capi, moe_forward, moe_forward_static) is host code only
+CO_SOURCES = ["moe_quant.hip", "moe_reduce.hip", "moe_gemm_mxfp4.hip", "moe_sort.hip", "moe_router.hip",
+              "moe_gemm_w4a16.hip", "moe_gemm_mxfp4_wide.hip"]
 
 
 def build_co(verbose=False, jobs=4):

@@ -86,16 +86,17 @@ __device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v
 // kernel issues NPF prefetch operations (sorted ids, activation DMA, scales) and 16 weight tiles.  They are spread
 // evenly instead of bunched: the texture-address path takes 16 clocks per 1 KB operation and CU, and a wave that finds
 // its queue full stalls at the issue, MFMAs included.
-//   prefetch operation k : gap pslot(k) % 3 of row group pslot(k) / 3, pslot(k) = k * NSLOT / NPF, NSLOT = 9 * MA
-//                          (the gaps 0..2 of the row groups of K-steps 0..2; K-step 3 leaves them time to land)
+//   prefetch operation k : gap pslot(k) % 3 of row group pslot(k) / 3, pslot(k) = k * NSLOT / NPF, NSLOT = 3 * PSTEPS * MA
+//                          (the gaps 0..2 of the row groups of K-steps 0 .. PSTEPS-1; the later K-steps leave them
+//                          time to land)
 //   weight tile (u, j)   : the registers are free once K-step u's MFMAs are issued: u < 3: gap 3 of row group
 //                          (u + 1) * MA + j * MA / 4; u = 3: after the last row group
 // The issue order is the same in every K-group (and in the prologue), which makes "all but the N youngest operations
 // have completed" exact: the functions below count N for the waits.
-template <int MA, int NPF>
+template <int MA, int NPF, int PSTEPS>
 struct VmSchedule
 {
-    static constexpr int NSLOT = 9 * MA;
+    static constexpr int NSLOT = 3 * PSTEPS * MA;
     static constexpr int TOTAL = NPF + 16;
     static constexpr int p_before_slot(int s)      // prefetch operations in slots < s
     {

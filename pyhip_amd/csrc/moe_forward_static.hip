@@ -20,7 +20,9 @@ int pyhip_moe_forward(const void*, int64_t, const uint8_t*, const uint8_t*, cons
 static __device__ __align__(256) unsigned char scratch[PYHIP_STATIC_SCRATCH_BYTES];
 
 // `scratch` names a host-side stand-in; the array's device address is asked for once per device, with that device
-// current, and only that address is ever handed to kernels
+// current, and only that address is ever handed to kernels.  Asking is what makes the runtime map the array on that
+// device, so it must not happen for the first time inside a stream capture: pyhip_moe_forward_static_capacity() asks
+// for the current device's address too, and is what a caller runs once per device while setting up.
 static void* scratch_device_ptr(int* rc_out)
 {
     static void* ptrs[64] = {nullptr};
@@ -50,7 +52,12 @@ static void* scratch_device_ptr(int* rc_out)
     return ptrs[dev];
 }
 
-extern "C" int64_t pyhip_moe_forward_static_capacity(void) { return PYHIP_STATIC_SCRATCH_BYTES; }
+extern "C" int64_t pyhip_moe_forward_static_capacity(void)
+{
+    int rc;
+    scratch_device_ptr(&rc);        // set-up for the current device; a failure is reported by the first real call
+    return PYHIP_STATIC_SCRATCH_BYTES;
+}
 
 extern "C" int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_row_stride, const uint8_t* w1,
                                         const uint8_t* w1_scale, const uint8_t* w2, const uint8_t* w2_scale,

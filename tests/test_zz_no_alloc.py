@@ -64,3 +64,68 @@ def test_static_scratch_entry_point_rejects_oversized_calls():
     rc = fn(one, 7168, one, one, one, one, None, None, one, one, None, None, one, 0, 8192, 8, 256, 7168, 2048, 128, 0, 0, 0,
             0.0, None)
     assert rc == 1 and b"scratch array holds" in lib.pyhip_moe_last_error()
+
+
+def _prepared_call(lib, L, dev_w, w4a16, bm):
+    """everything the static entry point needs, allocated up front; returns (call, out)"""
+    fn, cap = _static_fn(lib)
+    cap()                                         # maps the library's array on this device, outside any capture
+    w1, w1s, w2, w2s = dev_w
+    hidden = L.hidden.cuda()
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    out = torch.full((L.T, L.H), float("nan"), dtype=torch.bfloat16, device="cuda")
+    keep = (hidden, tw, ti, w1, w1s, w2, w2s)
+    args = (_lib.dptr(hidden), L.H, _lib.dptr(w1), _lib.dptr(w1s), _lib.dptr(w2), _lib.dptr(w2s), None, None,
+            _lib.dptr(ti), _lib.dptr(tw), None, None, _lib.dptr(out), 0, L.T, L.k, L.E, L.H, L.I, bm, w4a16, 0, 0, 0.0)
+
+    def call():
+        _lib.check(fn(*args, _lib.current_stream()), "moe_forward_static")
+    call.keep = keep
+    return call, out
+
+
+@pytest.mark.parametrize("w4a16", [0, 1])
+def test_static_scratch_entry_point_allocates_nothing(w4a16):
+    """device memory in use (the driver's count of free bytes and torch's own count) does not move across calls"""
+    lib = _lib.load()
+    L = cases.make_layer("dsv3_s", 24, seed=33)
+    call, out = _prepared_call(lib, L, cases.device_weights(L), w4a16, 16)
+    call()                                        # (first launch of these kernels in the process may load their code)
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("w4a16", [0, 1])
+def test_static_scratch_entry_point_under_graph_capture(w4a16):
+    """the call captured in a HIP graph and replayed, with eager work and synchronisations between the replays: every
+    replay must reproduce the eager result bit for bit"""
+    lib = _lib.load()
+    L = cases.make_layer("dsv3_s", 24, seed=34)
+    call, out = _prepared_call(lib, L, cases.device_weights(L), w4a16, 16)
+    call()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        call()                                    # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            call()
+    torch.cuda.current_stream().wait_stream(side)
+    for i in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), "replay %d differs" % i
+        scribble = torch.randn(1 << 20, device="cuda").sum()     # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(scribble)
