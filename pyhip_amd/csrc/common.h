@@ -102,6 +102,19 @@ __device__ __forceinline__ u32 amax15(u32 acc, u32 w)
     return acc > hi ? acc : hi;
 }
 
+// the same on packed halves: per 16-bit half, the larger magnitude pattern of a and b; amax15_fold joins the halves
+__device__ __forceinline__ u32 amax15x2(u32 a, u32 b)
+{
+    typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+    const v2us x = __builtin_bit_cast(v2us, a & 0x7FFF7FFFu), y = __builtin_bit_cast(v2us, b & 0x7FFF7FFFu);
+    return __builtin_bit_cast(u32, __builtin_elementwise_max(x, y));      // v_pk_max_u16
+}
+__device__ __forceinline__ u32 amax15_fold(u32 w)
+{
+    const u32 lo = w & 0xFFFFu, hi = w >> 16;
+    return lo > hi ? lo : hi;
+}
+
 // eight bf16 (one uint4) times a power of two -> eight e2m1 codes in one dword
 __device__ __forceinline__ u32 cvt8(uint4 v, float mul)
 {

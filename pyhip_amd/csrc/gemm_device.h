@@ -86,18 +86,21 @@ __device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v
 // kernel issues NPF prefetch operations (sorted ids, activation DMA, scales) and 16 weight tiles.  They are spread
 // evenly instead of bunched: the texture-address path takes 16 clocks per 1 KB operation and CU, and a wave that finds
 // its queue full stalls at the issue, MFMAs included.
-//   prefetch operation k : gap pslot(k) % 3 of row group pslot(k) / 3, pslot(k) = k * NSLOT / NPF, NSLOT = 3 * PSTEPS * MA
-//                          (the gaps 0..2 of the row groups of K-steps 0 .. PSTEPS-1; the later K-steps leave them
-//                          time to land)
+//   prefetch operation k : slot pslot(k) = k * NSLOT / NPF of the NSLOT = PGAPS * PSTEPS * MA slots that the last PGAPS of
+//                          the gaps 0..2 of the row groups of K-steps 0 .. PSTEPS-1 offer (the later K-steps leave
+//                          the operations time to land)
 //   weight tile (u, j)   : the registers are free once K-step u's MFMAs are issued: u < 3: gap 3 of row group
 //                          (u + 1) * MA + j * MA / 4; u = 3: after the last row group
 // The issue order is the same in every K-group (and in the prologue), which makes "all but the N youngest operations
 // have completed" exact: the functions below count N for the waits.
-template <int MA, int NPF, int PSTEPS>
+template <int MA, int NPF, int PSTEPS, int PGAPS = 3>
 struct VmSchedule
 {
-    static constexpr int NSLOT = 3 * PSTEPS * MA;
+    // prefetch operations use the last PGAPS of the gaps 0..2 of a row group (gap 0 also holds the LDS operand read)
+    static constexpr int NSLOT = PGAPS * PSTEPS * MA;
     static constexpr int TOTAL = NPF + 16;
+    static constexpr int slot_of(int n, int gap) { return n * PGAPS + gap - (3 - PGAPS); }      // gap >= 3 - PGAPS
+    static constexpr bool is_pgap(int gap) { return gap >= 3 - PGAPS && gap < 3; }
     static constexpr int p_before_slot(int s)      // prefetch operations in slots < s
     {
         const int c = (s * NPF + NSLOT - 1) / NSLOT;
@@ -112,19 +115,19 @@ struct VmSchedule
                 c += w_rg(u, j) < n;
         return c;
     }
-    static constexpr int before_rg(int n) { return p_before_slot(3 * n < NSLOT ? 3 * n : NSLOT) + w_before_rg(n); }
+    static constexpr int before_rg(int n) { return p_before_slot(PGAPS * n < NSLOT ? PGAPS * n : NSLOT) + w_before_rg(n); }
     static constexpr int w_index(int u, int j)
     {
         if(u == 3)
             return NPF + 12 + j;
         const int n = w_rg(u, j);
-        return p_before_slot(3 * (n + 1) < NSLOT ? 3 * (n + 1) : NSLOT) + 4 * u + j;
+        return p_before_slot(PGAPS * (n + 1) < NSLOT ? PGAPS * (n + 1) : NSLOT) + 4 * u + j;
     }
     // operations younger than the tiles of K-step u (issued one K-group ago) when K-step u starts
     static constexpr int younger(int u) { return TOTAL - 1 - w_index(u, 3) + before_rg(u * MA); }
     // operations younger than the last prefetch operation at the end of the K-group
     // (the weight tiles in gap 3 of its own row group come after it)
-    static constexpr int younger_end() { return 16 - w_before_rg(((NPF - 1) * NSLOT / NPF) / 3); }
+    static constexpr int younger_end() { return 16 - w_before_rg(((NPF - 1) * NSLOT / NPF) / PGAPS); }
 };
 
 template <int R>
@@ -250,10 +253,10 @@ __device__ __forceinline__ void gemm_zero_acc(v4f* xacc = nullptr)
         for(int i = 0; i < (16 * MT - 256) / 4; i++)
             xacc[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 }
-// the four accumulators of row group MTI, plus bias (bias4(j) = the address of the lane's four bf16 biases of weight
-// row group j; re-read per row group to keep the epilogue's register need small)
-template <int MT, int MTI, typename B>
-__device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4], B bias4, const v4f* xacc)
+// the four accumulators of row group MTI, plus bias when the instance has one (bias4(j) = the address of the lane's
+// four bf16 biases of weight row group j; re-read per row group to keep the epilogue's register need small)
+template <int MT, int MTI, bool BIAS, typename B>
+__device__ __forceinline__ void gemm_fetch_row(v4f (&row)[4], B bias4, const v4f* xacc)
 {
     static_for<4>([&](auto J) __attribute__((always_inline)) {
         constexpr int j = decltype(J)::value, a0 = (j * MT + MTI) * 4;
@@ -261,7 +264,7 @@ __device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4],
             row[j] = xacc[MTI - ACC_SPILL_MT0];
         else
             row[j] = (v4f){acc_fixed_read<a0>(), acc_fixed_read<a0 + 1>(), acc_fixed_read<a0 + 2>(), acc_fixed_read<a0 + 3>()};
-        if(g.bias)
+        if constexpr(BIAS)
         {
             const uint2 b = *(const uint2*)bias4(j);
             row[j][0] += bf16_bits_to_f32((uint16_t)b.x);
@@ -273,11 +276,18 @@ __device__ __forceinline__ void gemm_fetch_row(const GemmArgs& g, v4f (&row)[4],
 }
 // e, nt: (local) expert and weight tile; row0: sorted position of the wave's first row; wcol: which 64 (stage 1: 32 + 32)
 // of the tile's weight rows the wave owns; meta: the sorted ids of the wave's rows, their routing weights mpad words
-// further; ma: how many of the wave's row groups hold real rows (a prefix; may be <= 0)
-template <int STAGE, int MT, int ACT, bool ATOMIC>
+// further; ma: how many of the wave's row groups hold real rows (a prefix; may be <= 0).  BIAS: the layer has biases
+// (the kernel branches once per tile between the two instances).
+//
+// With one wave per SIMD (the tiles above 128 rows) nothing else runs while a wave is in its epilogue, so the row groups
+// are taken two at a time and everything up to the stores is one stretch of code without branches: the second group's
+// accumulator reads, conversions and lane exchanges fill the latencies of the first one's (the transcendental pipeline,
+// the exchanges).  The tiles up to 128 rows have two or more waves per SIMD for that, and no registers for a second group.
+template <int STAGE, int MT, int ACT, bool ATOMIC, bool BIAS>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, int row0, int wcol, const u32* meta, int mpad,
                                               int ma, int r, int kb, const v4f* xacc = nullptr)
 {
+    constexpr int PAIR = MT > 8 ? 2 : 1;
     const int I = g.N / 2;   // stage 1 only
     if(STAGE == 1)
     {
@@ -291,52 +301,74 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
         };
         // after the swap: lane rows 0..3 hold channel offsets 0, 16, 8, 24
         const int ch_out = chw + (kb & 1) * 16 + (kb >> 1) * 8;
-        static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
-            constexpr int mt = decltype(MTI)::value;
-            const int p = row0 + mt * 16 + r;
-            uint4 o     = make_uint4(0u, 0u, 0u, 0u);     // row groups that hold only padding store zeros
-            if(mt < ma)
+        const int blk = nt * 4 + wcol, jb = blk & 15;              // scale byte: see moe_quant.hip
+        const int s_col = (blk & ~15) + (jb & 3) * 4 + (jb >> 2);
+        static_for<(MT + PAIR - 1) / PAIR>([&](auto GI) __attribute__((always_inline)) {
+            constexpr int m0 = decltype(GI)::value * PAIR;
+            constexpr int NP = m0 + PAIR <= MT ? PAIR : MT - m0;       // row groups of this pair
+            uint4 o[NP];
+            u32 q4[NP], e8[NP];
+#pragma unroll
+            for(int q = 0; q < NP; q++)
+                o[q] = make_uint4(0u, 0u, 0u, 0u);                // row groups that hold only padding store zeros
+            if(m0 < ma)                                           // (a pair leaves together: a padding group next to a real one computes)
             {
-                v4f row[4];
-                gemm_fetch_row<MT, mt>(g, row, bz, xacc);
-                const bool ok = (int)(meta[mt * 16 + r] >> 24) < g.topk;
-                u32 d[2][2];
+                u32 ids[NP];
 #pragma unroll
-                for(int j = 0; j < 2; j++)
-                {
-                    float v[4];
+                for(int q = 0; q < NP; q++)
+                    ids[q] = meta[(m0 + q) * 16 + r];
+                static_for<NP>([&](auto Q) __attribute__((always_inline)) {
+                    constexpr int q = decltype(Q)::value, mt = m0 + q;
+                    v4f row[4];
+                    gemm_fetch_row<MT, mt, BIAS>(row, bz, xacc);
+                    u32 d[2][2];
 #pragma unroll
-                    for(int i = 0; i < 4; i++)
-                        v[i] = !ok ? 0.f : ACT == 0 ? silu_f32(row[j][i]) * row[j + 2][i] : swiglu_f32(row[j][i], row[j + 2][i], g.limit);
-                    d[j][0] = pack_bf16x2(v[0], v[1]);
-                    d[j][1] = pack_bf16x2(v[2], v[3]);
-                }
-                v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
-                v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
-                // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
-                o = make_uint4(t0.x, t1.x, t0.y, t1.y);
+                    for(int j = 0; j < 2; j++)
+                    {
+                        float v[4];
+#pragma unroll
+                        for(int i = 0; i < 4; i++)
+                            v[i] = ACT == 0 ? silu_f32(row[j][i]) * row[j + 2][i] : swiglu_f32(row[j][i], row[j + 2][i], g.limit);
+                        d[j][0] = pack_bf16x2(v[0], v[1]);
+                        d[j][1] = pack_bf16x2(v[2], v[3]);
+                    }
+                    v2u t0 = __builtin_amdgcn_permlane16_swap(d[0][0], d[1][0], false, false);
+                    v2u t1 = __builtin_amdgcn_permlane16_swap(d[0][1], d[1][1], false, false);
+                    // even lane rows: x = (kb, j0), y = (kb+1, j0); odd lane rows: x = (kb-1, j1), y = (kb, j1)
+                    const bool ok = (int)(ids[q] >> 24) < g.topk;          // padding rows store zeros
+                    o[q] = make_uint4(ok ? t0.x : 0u, ok ? t1.x : 0u, ok ? t0.y : 0u, ok ? t1.y : 0u);
+                });
             }
-            if(out)
-                *(uint4*)(out + (size_t)p * I + ch_out) = o;
+            // the wave's 32 channels of a row are exactly one MX block (8 channels in each of the four lane rows): block
+            // maximum across the lane rows, then the same arithmetic as the stand-alone quantiser (moe_quant.hip) on the
+            // bf16-rounded values, so both paths agree bit for bit
             if(g.out_q)
             {
-                // the wave's 32 channels of a row are exactly one MX block (8 channels in each of the four
-                // lane rows): block maximum across the lane rows, then the same arithmetic as the stand-alone
-                // quantiser (moe_quant.hip) on the bf16-rounded values, so both paths agree bit for bit
-                u32 am = amax15(amax15(amax15(amax15(0u, o.x), o.y), o.z), o.w);
-                v2u s16 = __builtin_amdgcn_permlane16_swap(am, am, false, false);
-                am      = s16.x > s16.y ? s16.x : s16.y;
-                v2u s32 = __builtin_amdgcn_permlane32_swap(am, am, false, false);
-                am      = s32.x > s32.y ? s32.x : s32.y;
-                const u32 e8 = mx_scale_byte(am);
-                *(u32*)(g.out_q + (size_t)p * (I / 2) + ch_out / 2) = cvt8(o, mx_inv_scale(e8));
-                if(kb == 0)
+#pragma unroll
+                for(int q = 0; q < NP; q++)
                 {
-                    const int blk = nt * 4 + wcol, jb = blk & 15;      // scale byte: see moe_quant.hip
-                    g.out_s[(size_t)p * g.OSK + (blk & ~15) + (jb & 3) * 4 + (jb >> 2)] = (uint8_t)e8;
+                    u32 am  = amax15_fold(amax15x2(amax15x2(o[q].x, o[q].y), amax15x2(o[q].z, o[q].w)));
+                    v2u s16 = __builtin_amdgcn_permlane16_swap(am, am, false, false);
+                    am      = s16.x > s16.y ? s16.x : s16.y;
+                    v2u s32 = __builtin_amdgcn_permlane32_swap(am, am, false, false);
+                    am      = s32.x > s32.y ? s32.x : s32.y;
+                    e8[q]   = mx_scale_byte(am);
+                    q4[q]   = cvt8(o[q], mx_inv_scale(e8[q]));
+                }
+#pragma unroll
+                for(int q = 0; q < NP; q++)
+                {
+                    const size_t p = (size_t)(row0 + (m0 + q) * 16 + r);
+                    *(u32*)(g.out_q + p * (I / 2) + ch_out / 2) = q4[q];
+                    if(kb == 0)
+                        g.out_s[p * g.OSK + s_col] = (uint8_t)e8[q];
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
+            if(out)
+#pragma unroll
+                for(int q = 0; q < NP; q++)
+                    *(uint4*)(out + (size_t)(row0 + (m0 + q) * 16 + r) * I + ch_out) = o[q];
+            __builtin_amdgcn_sched_barrier(0);      // a pair of row groups at a time: keeps the temporaries few
         });
     }
     else
@@ -346,46 +378,63 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
         uint16_t* out = (uint16_t*)g.out;
         const int chw = nt * 256 + wcol * 64;
         auto bz = [&](int j) __attribute__((always_inline)) { return g.bias + (size_t)e * g.N + chw + j * 16 + kb * 4; };
-        static_for<MT>([&](auto MTI) __attribute__((always_inline)) {
-            constexpr int mt = decltype(MTI)::value;
-            if(mt >= ma)
+        const int lane_col  = chw + kb * 16;
+        const u32 row_bytes = (u32)g.N * 2u;
+        static_for<(MT + PAIR - 1) / PAIR>([&](auto GI) __attribute__((always_inline)) {
+            constexpr int m0 = decltype(GI)::value * PAIR;
+            constexpr int NP = m0 + PAIR <= MT ? PAIR : MT - m0;
+            if(m0 >= ma)
                 return;
-            v4f row[4];
-            gemm_fetch_row<MT, mt>(g, row, bz, xacc);
-            const u32 id   = meta[mt * 16 + r];
-            const float rw = __builtin_bit_cast(float, meta[mpad + mt * 16 + r]);
-            const int tok = (int)(id & 0xFFFFFFu), slot = (int)(id >> 24);
-            const bool ok = slot < g.topk && tok < g.T;
-            u32 lo[4], hi[4];
+            u32 ids[NP], rws[NP];
 #pragma unroll
-            for(int j = 0; j < 4; j++)
+            for(int q = 0; q < NP; q++)
             {
-                lo[j] = pack_bf16x2(row[j][0] * rw, row[j][1] * rw);
-                hi[j] = pack_bf16x2(row[j][2] * rw, row[j][3] * rw);
+                ids[q] = meta[(m0 + q) * 16 + r];
+                rws[q] = meta[mpad + (m0 + q) * 16 + r];
             }
-            transpose4x4_rows(lo);
-            transpose4x4_rows(hi);
-            // lane row q now holds channels q*16 + c*4 .. +3 in (lo[c], hi[c])
-            if(ok && !ATOMIC)
-            {
-                // (plain stores: marked non-temporal they cost the down GEMM 5 % and the reduction, which then finds
-                // nothing of out3 in the last-level cache, another 4 %)
-                uint4* dst = (uint4*)(out + ((size_t)tok * g.topk + slot) * g.N + chw + kb * 16);
-                dst[0]     = make_uint4(lo[0], hi[0], lo[1], hi[1]);
-                dst[1]     = make_uint4(lo[2], hi[2], lo[3], hi[3]);
-            }
-            if(ok && ATOMIC)
-            {
-                typedef short v2s __attribute__((ext_vector_type(2)));
-                auto* dst = (__attribute__((address_space(1))) v2s*)(out + (size_t)tok * g.N + chw + kb * 16);
+            u32 lo[NP][4], hi[NP][4];
+            static_for<NP>([&](auto Q) __attribute__((always_inline)) {
+                constexpr int q = decltype(Q)::value, mt = m0 + q;
+                v4f row[4];
+                gemm_fetch_row<MT, mt, BIAS>(row, bz, xacc);
+                const float rw = __builtin_bit_cast(float, rws[q]);
 #pragma unroll
-                for(int c = 0; c < 4; c++)
+                for(int j = 0; j < 4; j++)
                 {
-                    __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c, __builtin_bit_cast(v2s, lo[c]));
-                    __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c + 1, __builtin_bit_cast(v2s, hi[c]));
+                    lo[q][j] = pack_bf16x2(row[j][0] * rw, row[j][1] * rw);
+                    hi[q][j] = pack_bf16x2(row[j][2] * rw, row[j][3] * rw);
+                }
+                transpose4x4_rows(lo[q]);
+                transpose4x4_rows(hi[q]);
+                // lane row c now holds channels c*16 + i*4 .. +3 in (lo[i], hi[i])
+            });
+#pragma unroll
+            for(int q = 0; q < NP; q++)
+            {
+                const u32 tok = ids[q] & 0xFFFFFFu, slot = ids[q] >> 24;
+                const bool ok = (int)slot < g.topk && (int)tok < g.T;       // (a padding group next to a real one: all false)
+                if(ok && !ATOMIC)
+                {
+                    // (plain stores: marked non-temporal they cost the down GEMM 5 % and the reduction, which then finds
+                    // nothing of out3 in the last-level cache, another 4 %)
+                    const u32 orow = tok * (u32)g.topk + slot;              // row of out3 [tokens * topk, N]
+                    uint4* dst = (uint4*)((unsigned long long)(out + lane_col) + (unsigned long long)orow * row_bytes);
+                    dst[0]     = make_uint4(lo[q][0], hi[q][0], lo[q][1], hi[q][1]);
+                    dst[1]     = make_uint4(lo[q][2], hi[q][2], lo[q][3], hi[q][3]);
+                }
+                if(ok && ATOMIC)
+                {
+                    typedef short v2s __attribute__((ext_vector_type(2)));
+                    auto* dst = (__attribute__((address_space(1))) v2s*)((unsigned long long)(out + lane_col) + (unsigned long long)tok * row_bytes);
+#pragma unroll
+                    for(int c = 0; c < 4; c++)
+                    {
+                        __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c, __builtin_bit_cast(v2s, lo[q][c]));
+                        __builtin_amdgcn_global_atomic_fadd_v2bf16(dst + 2 * c + 1, __builtin_bit_cast(v2s, hi[q][c]));
+                    }
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);      // one row group at a time: keeps the temporaries few
+            __builtin_amdgcn_sched_barrier(0);      // a pair of row groups at a time: keeps the temporaries few
         });
     }
 }

@@ -336,18 +336,27 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     v4f xacc[TALL ? MT - ACC_SPILL_MT0 : 1];      // the accumulator tiles beyond the accumulation registers (288-row tile)
     auto zero_acc = [&]() __attribute__((always_inline)) { gemm_zero_acc<MT>(xacc); };
     auto epilogue = [&](const TileId& t, const u32* meta, int ma_t) __attribute__((always_inline)) {
-        gemm_epilogue<STAGE, MT, ACT, ATOMIC>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
+        if(g.bias)
+            gemm_epilogue<STAGE, MT, ACT, ATOMIC, true>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
+        else
+            gemm_epilogue<STAGE, MT, ACT, ATOMIC, false>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
     };
 
     // ---------------------------------------------------------------- pipeline
     constexpr int MA = MT;                    // row groups that take part in the MFMAs
-    // One wave per SIMD (the tiles above 128 rows): the K-group's prefetches are spread over three K-steps and every
-    // instruction that is not an MFMA sits in a gap between two MFMAs.  Two or more waves per SIMD fill each other's
-    // gaps: there the four MFMAs of a row group stay back to back, the other instructions follow them, and the
-    // prefetches all go out during K-step 0 (measured against the spread form at 128 rows: gpt-oss shape, 4096 tokens,
-    // layer 0.573 against 0.597 ms; Mixtral shape, 512 tokens, 0.216 against 0.224 ms).
+    // One wave per SIMD (the tiles above 128 rows): the K-group's prefetches are spread over two K-steps and every
+    // instruction that is not an MFMA sits in a gap between two MFMAs.  (Measured per K-step of the 288-row tile,
+    // DeepSeek-V3 shape, 8192 tokens, in clocks, 1152 being the MFMAs alone: a K-step that only issues its four weight
+    // tiles takes 1275-1300; every LDS-DMA operation adds about 40 wherever it sits, which gap of the row group included:
+    // all 29 in K-step 0: 2705 + 3 x 1300; over two K-steps 1700 + 1950 + 2 x 1290; over three 1545 + 1770 + 1790 + 1275.
+    // The same loads into registers instead of LDS add 10 each: the cost is in the DMA's write to LDS, not in the
+    // fetch.  Two K-steps leave the last operation a K-step and a half to land before the barrier.)
+    // Two or more waves per SIMD fill each other's gaps: there the four MFMAs of a row group stay back to back, the
+    // other instructions follow them, and the prefetches all go out during K-step 0 (measured against the spread form
+    // at 128 rows: gpt-oss shape, 4096 tokens, layer 0.573 against 0.597 ms; Mixtral shape, 512 tokens, 0.216 against
+    // 0.224 ms).
     constexpr bool SPREAD = MT > 8;
-    using VS = VmSchedule<MA, NPF, SPREAD ? 3 : 1>;
+    using VS = VmSchedule<MA, NPF, SPREAD ? 2 : 1>;
     static_assert(VS::younger(0) <= 63 && VS::younger(1) <= 63 && VS::younger(2) <= 63 && VS::younger(3) <= 63,
                   "the vector-memory counter has six bits");
     // sorted ids and routing weights of a tile's rows -> LDS meta buffer `buf` (DMA, 64 rows per operation, spread over
@@ -393,9 +402,9 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
         constexpr int n = decltype(N)::value, gp = decltype(G)::value;
         if constexpr(gp < 3)
         {
-            if constexpr(3 * n + gp < VS::NSLOT)
+            if constexpr(VS::is_pgap(gp) && VS::slot_of(n, gp) < VS::NSLOT)
             {
-                constexpr int k0 = VS::p_before_slot(3 * n + gp), k1 = VS::p_before_slot(3 * n + gp + 1);
+                constexpr int k0 = VS::p_before_slot(VS::slot_of(n, gp)), k1 = VS::p_before_slot(VS::slot_of(n, gp) + 1);
                 static_for<k1 - k0>([&](auto Q) __attribute__((always_inline)) {
                     prefetch_op(std::integral_constant<int, k0 + decltype(Q)::value>{}, TS, kpre);
                 });

@@ -254,8 +254,12 @@ __global__ void __launch_bounds__(WIDE_THREADS) moe_gemm_mxfp4_wide_kernel(GemmA
     // accumulators and epilogue: gemm_device.h (a wave's rows start wr * 128 rows into the tile)
     auto zero_acc = [&]() __attribute__((always_inline)) { gemm_zero_acc<MT>(); };
     auto epilogue = [&](const TileId& t, const u32* meta, int ma_t) __attribute__((always_inline)) {
-        gemm_epilogue<STAGE, MT, ACT, false>(g, t.e, t.nt, t.m_blk * BM + wr * MT * 16, wc, meta + wr * MT * 16, MPAD,
-                                              ma_t - wr * MT, r, kb);
+        if(g.bias)
+            gemm_epilogue<STAGE, MT, ACT, false, true>(g, t.e, t.nt, t.m_blk * BM + wr * MT * 16, wc, meta + wr * MT * 16, MPAD,
+                                                        ma_t - wr * MT, r, kb);
+        else
+            gemm_epilogue<STAGE, MT, ACT, false, false>(g, t.e, t.nt, t.m_blk * BM + wr * MT * 16, wc, meta + wr * MT * 16, MPAD,
+                                                         ma_t - wr * MT, r, kb);
     };
 
     // ---------------------------------------------------------------- pipeline
