@@ -113,14 +113,23 @@ extern "C" int pyhip_moe_pick_block_m(int64_t tokens, int topk, int experts, int
         return 64;
     // Prefill sizes: 128 rows, except where a taller tile lets nearly every expert fit ONE row block, so that each weight
     // tile is read once instead of two or three times.  The tiles above 128 rows run one wave per SIMD and have a long
-    // epilogue, which only pays with a long K loop (hidden >= 6144); the gpt-oss, Qwen3 and Mixtral shapes (hidden 3072 /
-    // 4096) lose 1-13 % with them at the same rows per expert.  DeepSeek-V3 shape, whole layer, ms, tiles of 128 / 160 /
+    // epilogue, which pays most with a long K loop (hidden >= 6144).  DeepSeek-V3 shape, whole layer, ms, tiles of 128 / 160 /
     // 192 / 256 / 288 rows by expected rows per expert (between machines the order of close neighbours can flip):
     //    96: 1.28 / 1.33 / 1.36 / 1.50 /  -       160: 2.26 / 1.93 / 1.49 / 1.60 / 1.73      232: 1.97 /  -   /  -   / 1.86 / 1.92
     //   104: 1.36 / 1.35 / 1.38 / 1.52 / 1.66     168: 2.08 / 2.22 / 1.55 / 1.62 / 1.75      240: 2.09 /  -   /  -   / 1.96 / 1.94
     //   120: 1.50 / 1.37 / 1.40 / 1.51 / 1.63     176: 2.04 / 2.63 / 1.65 / 1.64 / 1.77      256: 2.26 /  -   /  -   / 2.64 / 2.02
     //   128: 1.72 / 1.39 / 1.42 / 1.53 / 1.65     192: 1.92 / 2.67 / 2.20 / 1.68 / 1.81      272: 2.46 /  -   /  -   / 3.29 / 2.36
     //   136: 1.92 / 1.43 / 1.43 / 1.54 / 1.67     208: 1.91 /  -   /  -   / 1.72 / 1.85      288: 2.57 /  -   /  -   / 3.53 / 2.97
+    // With the shorter K loop of hidden 3072 / 4096 only the first step pays, and only under an even router: 100-132
+    // expected rows per expert, where the 128-row tile needs a second, nearly empty block for half of the experts (whole
+    // layer, ms, 128 / 160 / 192 / 256 rows: Mixtral shape, 512 tokens: 0.210 / 0.191 / 0.198 / 0.216; gpt-oss shape, 4096
+    // tokens: 0.564 / 0.499 / 0.513 / 0.556; the Qwen3 shape's Zipf router at 2048 tokens, the same mean: 0.399 / 0.420 /
+    // 0.425 / 0.452: most of its experts are far below the mean and pay for the taller tile's empty row groups).  Further
+    // up, the taller tiles win by 3-11 % under the even routers at exactly the sizes where an expert fills one block
+    // (192 rows at 160 per expert, 288 at 256) and lose up to 20 % under the uneven one and between those sizes: left at
+    // 128 rows.
+    if(hidden < 6144 && est >= 100 && est <= 132)
+        return 160;
     if(hidden >= 6144)
     {
         if(est >= 100 && est <= 132)

@@ -282,20 +282,25 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             wrs[0] = wrs[1] = make_rsrc(g.w + row * Kb, (u32)(64 * Kb));
             wsrs[0] = wsrs[1] = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)(2 * sc_tile));
         }
+        // (all the reads first, from a clamped position and without a branch between them: one LDS round trip instead of
+        // one per slot)
+        u32 idv[NA];
 #pragma unroll
         for(int i = 0; i < NA; i++)
         {
             const int slot = wave + 4 * i;
-            int row        = -1;                     // padding rows and unused slots fetch nothing
-            if(slot < MT)
-            {
-                const u32 id  = ids[slot * 16 + dma_row];
-                const int tok = (int)(id & 0xFFFFFFu);
-                if((int)(id >> 24) < g.topk && tok < g.T)
-                    row = STAGE == 1 ? tok : t.m_blk * BM + slot * 16 + dma_row;
-            }
-            a_off[i]  = row < 0 ? (int)OOB : row * Kb + dma_chunk * 16;
-            as_off[i] = row < 0 ? (int)OOB : row * g.SK + (lane & 3) * 4;
+            idv[i]         = ids[(slot < MT ? slot : MT - 1) * 16 + dma_row];
+        }
+#pragma unroll
+        for(int i = 0; i < NA; i++)
+        {
+            const int slot = wave + 4 * i;
+            const int tok  = (int)(idv[i] & 0xFFFFFFu);
+            // padding rows and unused slots fetch nothing
+            const bool ok  = slot < MT && (int)(idv[i] >> 24) < g.topk && tok < g.T;
+            const int row  = STAGE == 1 ? tok : t.m_blk * BM + slot * 16 + dma_row;
+            a_off[i]       = ok ? row * Kb + dma_chunk * 16 : (int)OOB;
+            as_off[i]      = ok ? row * g.SK + (lane & 3) * 4 : (int)OOB;
         }
     };
 

@@ -88,9 +88,10 @@ def pick_block_m(tokens, topk, experts, hidden=0, w4a16=False):
     The tiles of 160, 192, 256 and 288 rows (one wave per SIMD, slower per FLOP) are taken where they save whole passes
     over the weights: where a 128-row tile needs two or three blocks for most experts and the taller tile one, read with
     non-temporal loads (100-132 expected rows per expert: 160 rows; up to 172: 192; up to 236: 256; up to 276: 288).
-    Their long epilogue only pays with a long K loop: DS-V3 (hidden 7168) T = 4096 / 6144: 1.39 / 1.68 ms against
-    1.72 / 1.92 ms with 128 rows, T = 8192: 2.02-2.06 ms with 288 rows against 2.26-2.29; the gpt-oss, Qwen3 and Mixtral shapes
-    (hidden 3072 / 4096) lose 1-13 % with them at the same rows per expert."""
+    Their long epilogue pays most with a long K loop: DS-V3 (hidden 7168) T = 4096 / 6144: 1.36 / 1.64 ms against
+    1.70 / 1.92 ms with 128 rows, T = 8192: 1.95 ms with 288 rows against 2.26; at hidden 3072 / 4096 only the 160-row step
+    is taken (100-132 expected rows per expert: gpt-oss shape T = 4096 0.50 against 0.56 ms, Mixtral shape T = 512 0.19
+    against 0.21; a router that loads its experts unevenly loses with it: Qwen3 shape, Zipf, T = 2048 0.42 against 0.40)."""
     return int(_lib.load().pyhip_moe_pick_block_m(tokens, topk, experts, hidden, 1 if w4a16 else 0))
 
 
