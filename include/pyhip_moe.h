@@ -145,7 +145,11 @@ int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint
  *   a2_q/a2_scale  quantised stage-1 output [n_blk*block_m, inter/2] / scales (sorted-row order)
  *   w2, w2_scale   u8 [experts, hidden, inter/2] pre-shuffled; e8m0 shuffled over [experts*hidden, inter/32]
  *   bias2          bf16 [experts, hidden] or NULL (added before the routing weight)
- *   out3           bf16 [tokens, topk, hidden]; only (token, slot) pairs that were sorted are written
+ *   out3           bf16 [tokens, topk, hidden]; only (token, slot) pairs that were sorted are written: the slots of
+ *                  pairs the sort dropped (expert id outside [0, experts), masked expert, token past the local
+ *                  count) keep whatever the buffer held.  Reduce with pyhip_moe_topk_reduce_routed, which leaves
+ *                  those slots out by the same rule, or clear out3 first when the plain pyhip_moe_topk_reduce is
+ *                  used with a routing that drops pairs.
  * inter % 512 == 0, hidden % 256 == 0. */
 int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
                           const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
@@ -209,7 +213,9 @@ int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t*
  * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.
  * Replaces moe_gemm_final_reduce_bf16, src/contrib/moe_gemm_mxfp4.py:199-282
  * (launch: tests/contrib/moe/test_moe.py:764-771).  out is bf16 or (out_is_f32 != 0) fp32.
- * num_valid_ids (may be NULL): when given, only tokens < num_valid_ids[1] are reduced. */
+ * num_valid_ids (may be NULL): when given, only tokens < num_valid_ids[1] are reduced.
+ * Every slot of in[] is read: after a sort that dropped pairs (expert_mask, ids out of range) the down GEMMs have
+ * left those slots unwritten, so either in[] was cleared before the GEMM or pyhip_moe_topk_reduce_routed is used. */
 int pyhip_moe_topk_reduce(const void* in_bf16, void* out, int64_t tokens, int topk, int hidden, int out_is_f32,
                           const uint32_t* num_valid_ids, pyhip_stream_t stream);
 

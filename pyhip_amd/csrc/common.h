@@ -40,6 +40,15 @@ extern "C" void pyhip_set_error(const char* fmt, ...);
         }                                                                         \
     } while(0)
 
+// Which (token, slot) pairs take part in the layer: the expert id names an expert (0 <= e < experts) that the
+// expert mask, when there is one, does not switch off.  The routing sort drops every other pair, the down GEMMs
+// then never write that pair's slot of out3, and the routing-aware top-k reduction leaves the slot out: all three
+// by this one rule.  (Tokens past num_local_tokens are dropped as whole rows by the callers' token limits.)
+__device__ __forceinline__ bool moe_pair_is_kept(int e, int experts, const int* expert_mask)
+{
+    return e >= 0 && e < experts && (!expert_mask || expert_mask[e] != 0);
+}
+
 __device__ __forceinline__ u32 pack_bf16x2(float a, float b)
 {
     v2f v = {a, b};

@@ -50,7 +50,7 @@ __global__ void __launch_bounds__(256)
                 if(ROUTED && on[j])
                 {
                     const int e = t < T_local ? rt.topk_ids[t * k + s0 + j] : -1;
-                    on[j]       = e >= 0 && e < rt.experts && (!rt.expert_mask || rt.expert_mask[e] != 0);
+                    on[j]       = moe_pair_is_kept(e, rt.experts, rt.expert_mask);
                 }
             }
 #pragma unroll

@@ -91,9 +91,7 @@ struct WavePairs
 #pragma unroll
         for(int g = 0; g < NG; g++)
         {
-            if(e[g] >= a.E)
-                e[g] = -1;
-            if(a.expert_mask && e[g] >= 0 && a.expert_mask[e[g]] == 0)
+            if(!moe_pair_is_kept(e[g], a.E, a.expert_mask))
                 e[g] = -1;
         }
     }
@@ -182,7 +180,7 @@ __device__ __forceinline__ u32 expert_offsets(const SortArgs& a, const u32* tot,
     for(int e0 = 0; e0 < a.E; e0 += blockDim.x)
     {
         int e     = e0 + threadIdx.x;
-        bool on   = e < a.E && (!a.expert_mask || a.expert_mask[e] != 0);
+        bool on   = moe_pair_is_kept(e, a.E, a.expert_mask);
         u32 pad   = (on && e < a.E) ? (tot[e] + a.Bm - 1) / a.Bm * a.Bm : 0u;
         u32 one   = on ? 1u : 0u;
         // inclusive scan inside the wave (two values packed: padded size, mask count)
@@ -248,7 +246,7 @@ __device__ __forceinline__ void fill_blocks(const SortArgs& a, const u32* tot, c
     const u32 tid = threadIdx.x, nthreads = blockDim.x;
     for(u32 e = tid / 16; e < (u32)a.E; e += nthreads / 16)
     {
-        if(tot[e] == 0 || (a.expert_mask && a.expert_mask[e] == 0))
+        if(tot[e] == 0 || !moe_pair_is_kept((int)e, a.E, a.expert_mask))
             continue;
         const u32 b0 = off[e] / a.Bm, b1 = b0 + (tot[e] + a.Bm - 1) / a.Bm;
         for(u32 b = b0 + tid % 16; b < b1; b += 16)

@@ -4,12 +4,14 @@
 (tests/contrib/moe/test_fused_moe.py:38,87): softmax over the experts, top-k, optional renormalisation.
 ``grouped_topk`` is DeepSeek-V3's routing (sigmoid scores, ``num_expert_group`` groups of consecutive experts,
 the ``topk_group`` groups with the largest sum of their two best scores stay, top-k inside them).
+``append_shared_experts`` turns experts that every token visits (DeepSeek-V3 has one) into extra routing slots, so
+that the grouped GEMMs compute them in the same launches as the routed experts.
 """
 import torch
 
 from . import _lib
 
-__all__ = ["fused_topk", "grouped_topk"]
+__all__ = ["fused_topk", "grouped_topk", "append_shared_experts"]
 
 
 def _scores(gating_output, pad_ok):
@@ -49,3 +51,20 @@ def grouped_topk(gating_output, topk, renormalize=True, num_expert_group=8, topk
                                                   1 if renormalize else 0, _lib.dptr(w), _lib.dptr(ids),
                                                   _lib.current_stream()), "topk_grouped_sigmoid")
     return w, ids
+
+
+def append_shared_experts(topk_weights, topk_ids, num_routed_experts, num_shared_experts=1, shared_weight=1.0):
+    """Routing for a layer whose weight tensors hold ``num_shared_experts`` shared experts behind the
+    ``num_routed_experts`` routed ones (``w1`` [E + S, 2I, H/2], ``w2`` [E + S, H, I/2]): every token gets S more
+    slots, slot ``k + s`` naming expert ``E + s`` with weight ``shared_weight``.  The layer then computes
+    ``sum_k w_k * expert_k(x) + shared_weight * sum_s shared_s(x)`` in one pass: to the sort and the GEMMs a shared
+    expert is an expert that happens to receive every token (T rows, T / block_size row blocks), and the top-k
+    reduction adds its slot last, in fp32, before the one rounding of the output.
+    -> (topk_weights f32 [T, k + S], topk_ids i32 [T, k + S]) on the inputs' device."""
+    assert topk_ids.dim() == 2 and topk_weights.shape == topk_ids.shape and num_shared_experts >= 1
+    T = topk_ids.shape[0]
+    ids = torch.arange(num_routed_experts, num_routed_experts + num_shared_experts, dtype=torch.int32,
+                       device=topk_ids.device).expand(T, num_shared_experts)
+    w = torch.full((T, num_shared_experts), float(shared_weight), dtype=torch.float32, device=topk_weights.device)
+    return (torch.cat([topk_weights.float(), w], dim=1).contiguous(),
+            torch.cat([topk_ids.to(torch.int32), ids], dim=1).contiguous())

@@ -101,7 +101,13 @@ def test_row_block_heuristic():
     assert pick_block_m(7680, 8, 256, 7168) == 288 and pick_block_m(8192, 8, 256, 7168) == 288
     assert pick_block_m(8832, 8, 256, 7168) == 288 and pick_block_m(8864, 8, 256, 7168) == 128
     assert pick_block_m(8192, 8, 256, 7168, True) == 64
-    assert pick_block_m(4096, 4, 128, 3072) == 128 and pick_block_m(2048, 8, 128, 4096) == 128
+    # short K loop: 160 rows where one such block holds an expert that would need a second, nearly empty 128-row block
+    # (100 to 132 expected rows per expert), 128 rows otherwise
+    assert pick_block_m(4096, 4, 128, 3072) == 160 and pick_block_m(2048, 8, 128, 4096) == 160
+    assert pick_block_m(512, 2, 8, 4096) == 160 and pick_block_m(4096, 2, 8, 4096) == 128
+    assert pick_block_m(1584, 8, 128, 4096) == 128 and pick_block_m(1600, 8, 128, 4096) == 160     # 99 / 100
+    assert pick_block_m(2112, 8, 128, 4096) == 160 and pick_block_m(2128, 8, 128, 4096) == 128     # 132 / 133
+    assert pick_block_m(8192, 8, 128, 4096) == 128
 
 
 def test_auto_method_rule():

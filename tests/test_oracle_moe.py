@@ -131,3 +131,28 @@ def test_swiglu_pins():
     gv, uv = np.minimum(4 * x.astype(np.float64), 5.0), np.clip(2 * x.astype(np.float64), -5.0, 5.0)
     np.testing.assert_allclose(got, mxfp4.bf16_round(closed(gv, uv).astype(np.float32)), rtol=2 ** -7, atol=1e-6)
     assert np.abs(got - moe.gateup_ref(x, w1)).max() > 0.1                                             # differs from SiLU
+
+
+@pytest.mark.parametrize("act", ["a4", "a16"])
+def test_shared_expert_as_an_extra_slot_is_routed_plus_dense(act):
+    """A shared expert appended as slot k (pyhip_amd.routing.append_shared_experts) gives the routed experts' sum plus
+    the shared expert applied to every token: checked on the oracle by evaluating the two halves separately."""
+    from pyhip_amd.routing import append_shared_experts
+    rng = np.random.default_rng(5)
+    E, T, k, H, I = 4, 11, 2, 64, 32
+    hidden, w1q, w1s, w2q, w2s, _, _ = _layer(rng, E + 1, T, k, H, I)
+    tw, ti = routing.softmax_topk(rng.standard_normal((T, E)), k)          # routed experts 0 .. E-1 only
+    tw2, ti2 = append_shared_experts(torch.from_numpy(tw), torch.from_numpy(ti), E, 1, shared_weight=0.5)
+    assert tw2.dtype == torch.float32 and ti2.dtype == torch.int32 and tw2.shape == ti2.shape == (T, k + 1)
+    assert (ti2[:, :k].numpy() == ti).all() and (ti2[:, k] == E).all()
+    assert (tw2[:, :k].numpy() == tw).all() and (tw2[:, k] == 0.5).all()
+    both = moe.moe_ref(hidden, w1q, w1s, w2q, w2s, tw2.numpy(), ti2.numpy(), act=act)
+    routed = moe.moe_ref(hidden, w1q[:E], w1s[:E], w2q[:E], w2s[:E], tw, ti, act=act)
+    x = moe.act_quant_dequant(hidden) if act == "a4" else hidden
+    a2 = moe.gateup_ref(x, moe.expert_weights_f32(w1q[E], w1s[E]))
+    a2 = moe.act_quant_dequant(a2) if act == "a4" else a2
+    shared = moe.down_ref(a2, moe.expert_weights_f32(w2q[E], w2s[E]), np.full(T, 0.5, np.float32))
+    assert (both == routed + shared).all()           # the shared slot is added last, in fp32: the same operations
+    # two shared experts
+    tw3, ti3 = append_shared_experts(torch.from_numpy(tw), torch.from_numpy(ti), E - 1, 2)
+    assert (ti3[:, k:] == torch.tensor([E - 1, E], dtype=torch.int32)).all() and (tw3[:, k:] == 1.0).all()
