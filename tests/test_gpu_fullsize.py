@@ -140,8 +140,13 @@ def test_sampled_experts_and_properties(layer, T, method):
         assert cos >= 0.999 and cd <= 0.01
         assert err_g.max() <= 1e-2 * rms
         if a4 and nflip:
-            # a stage-1 value that sits on a bf16 rounding boundary AND on an e2m1 boundary moves one re-quantised
-            # activation by a whole e2m1 step (tests/test_gpu_moe.py::_end_to_end): isolated outliers, bounded
+            # a stage-1 value that sits on a bf16 rounding boundary AND on an e2m1 (or block-scale) boundary moves a
+            # re-quantised activation by a whole e2m1 step (tests/test_gpu_moe.py::_end_to_end).  Only the rows where
+            # that happened (the kernel's stage-1 row re-quantises differently from the oracle's) may exceed the
+            # strict bound, they stay isolated and bounded; every other row meets the strict bound.
+            moved = (moe.act_quant_dequant(got_a2) != moe.act_quant_dequant(a2)).any(axis=1)
+            row_err = err.max(axis=1)
+            assert row_err[~moved].max(initial=0.0) <= 1e-2 * rms, "an outlier in a row whose stage-1 result re-quantises as the oracle's"
             assert np.mean(err > 1e-2 * rms) <= 2e-3 and err.max() <= 0.1 * rms
         else:
             assert err.max() <= 1e-2 * rms
