@@ -171,12 +171,15 @@ def stage_pass(torch, fused_moe, W, res, block_m, method, passes=8):
     return {k: sum(v) / len(v) for k, v in acc.items()}
 
 
-def epilogue_comparison(torch, fused_moe, W, res, block_m):
-    """the tail of the layer both ways, from events in untimed passes of the step-by-step path: down GEMM storing
-    out3[T, k, H] + top-k reduction (deterministic, the product path) against output clear + down GEMM with packed
-    bf16 atomics into out[T, H] (the reference's atomic variant)"""
-    r = {}
-    for mode in ("store", "atomic"):
+def epilogue_comparison(torch, fused_moe, W, res, block_m, modes=("store", "atomic", "last_arriver")):
+    """the tail of the layer three ways, from events in untimed passes of the step-by-step path: down GEMM storing
+    out3[T, k, H] + top-k reduction (deterministic, the product path); output clear + down GEMM with packed bf16
+    atomics into out[T, H] (the reference's atomic variant); counter set-up + down GEMM whose workgroups also sum a
+    token's slots, whoever stores the last one (deterministic, bit-identical to the first)"""
+    names = {"store": "down_gemm_store_plus_reduce_ms", "atomic": "clear_plus_down_gemm_atomic_ms",
+             "last_arriver": "setup_plus_down_gemm_last_arriver_ms"}
+    r = {"block_m": block_m}
+    for mode in modes:
         kw = call_kwargs(W, block_m, "a4w4")
         events = []
         for i in range(10):
@@ -187,8 +190,8 @@ def epilogue_comparison(torch, fused_moe, W, res, block_m):
         for name, a, b in events:
             acc.setdefault(name, []).append(a.elapsed_time(b))
         acc = {k: sum(v) / len(v) for k, v in acc.items()}
-        r[mode] = round(acc["gemm2"] + acc.get("reduce", 0.0), 4)
-    return {"down_gemm_store_plus_reduce_ms": r["store"], "clear_plus_down_gemm_atomic_ms": r["atomic"]}
+        r[names[mode]] = round(acc["gemm2"] + acc.get("reduce", 0.0), 4)
+    return r
 
 
 def tile256_comparison(torch, fused_moe, W, shape, tokens):
@@ -379,6 +382,8 @@ def main():
             epi = None
             if a.epilogue_comparison:
                 epi = {"tokens_%d" % a.tokens: epilogue_comparison(torch, fused_moe, W, main_res, 128),
+                       "tokens_%d_rows_288" % a.tokens: epilogue_comparison(torch, fused_moe, W, main_res, 288,
+                                                                            ("store", "last_arriver")),
                        "tokens_%d" % a.decode_tokens: epilogue_comparison(torch, fused_moe, W, dec, 16)}
         del W
         torch.cuda.empty_cache()

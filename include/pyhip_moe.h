@@ -187,6 +187,24 @@ int pyhip_moe_gemm2_mxfp4_atomic(const uint8_t* a2_q, const uint8_t* a2_scale, c
                                  int topk, int experts, int hidden, int inter, int block_m, int64_t n_blk,
                                  pyhip_stream_t stream);
 
+/* Stage 2 with the top-k reduction done inside it, deterministically: out3 is written as by pyhip_moe_gemm2_mxfp4, and the
+ * workgroup that stores the last of a token's slots for a 256-channel weight tile sums that token's slots in fp32 in
+ * slot order and writes out[tokens, hidden] (bf16, or fp32 when out_is_f32 != 0): the arithmetic of
+ * pyhip_moe_topk_reduce_routed, so the same bits whatever the arrival order, with no reduction launch and no waiting
+ * between workgroups.  The deterministic counterpart of the reference's atomic epilogue
+ * (src/contrib/moe_gemm_mxfp4.py:1334-1398); pyhip_moe_forward keeps the two-kernel path, which measures faster at
+ * prefill sizes.
+ *   topk_ids, expert_mask, num_local_tokens   the routing as given to the sort (for the drop rule)
+ *   arrive        int32 [tokens * hidden / 256], scratch (initialised by this call)
+ * block_m 16, 128 or 288. */
+int pyhip_moe_gemm2_mxfp4_reduce(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
+                                 const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
+                                 const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
+                                 const uint32_t* schedule, void* out3_bf16, const int32_t* topk_ids,
+                                 const int32_t* expert_mask, const int32_t* num_local_tokens, int32_t* arrive, void* out,
+                                 int out_is_f32, int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                 int64_t n_blk, pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * The same two GEMMs with bf16 activations ("w4a16"): weights are expanded from MXFP4 to bf16 in registers
  * and multiplied with the bf16 MFMA; nothing is quantised at run time.  Replaces moe_2stage_splitk with fp4

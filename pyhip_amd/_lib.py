@@ -42,6 +42,8 @@ SIGNATURES = {
     "pyhip_moe_gemm1_mxfp4_lds": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _F, _P]),
     "pyhip_moe_gemm2_mxfp4_lds": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _P]),
     "pyhip_moe_gemm2_mxfp4_atomic": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
+    "pyhip_moe_gemm2_mxfp4_reduce": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I,
+                                          _I, _I, _I, _I, _I, _I, _L, _P]),
     "pyhip_moe_gemm1_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _P]),
     "pyhip_moe_gemm2_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _P]),
     "pyhip_moe_topk_reduce": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),

@@ -21,7 +21,10 @@ class GemmArgs(ctypes.Structure):
     _fields_ = [("a_q", _P), ("a_s", _P), ("w", _P), ("w_s", _P), ("bias", _P), ("sorted_ids", _P), ("sorted_w", _P),
                 ("sorted_e", _P), ("num_valid", _P), ("sched", _P), ("out", _P), ("out_q", _P), ("out_s", _P),
                 ("OSK", _I), ("limit", _F), ("T", _I), ("topk", _I), ("K", _I), ("N", _I), ("SK", _I), ("SC", _I),
-                ("n_blk", _I), ("n_tiles", _I), ("a_rows", _I), ("E", _I)]
+                ("n_blk", _I), ("n_tiles", _I), ("a_rows", _I), ("E", _I),
+                # STAGE 3 (down GEMM with the last-arriver reduction) only
+                ("arrive", _P), ("topk_ids", _P), ("expert_mask", _P), ("final_out", _P), ("final_f32", _I),
+                ("experts_all", _I)]
 
 
 class QuantArgs(ctypes.Structure):

@@ -26,6 +26,12 @@ struct GemmArgs
     int OSK;
     float limit;               // stage 1, SwiGLU: the clamp
     int T, topk, K, N, SK, SC, n_blk, n_tiles, a_rows, E;
+    // stage 3 only (the down GEMM that also reduces over the slots, see gemm_arrive_reduce)
+    int* arrive            = nullptr;   // [T, n_tiles] slots of the token that have not been stored yet
+    const int* topk_ids    = nullptr;   // [T, topk] the routing ...
+    const int* expert_mask = nullptr;   // ... and the expert mask ([experts_all] or null), for the drop rule
+    void* final_out        = nullptr;   // [T, N] bf16, or fp32 when final_f32 != 0
+    int final_f32 = 0, experts_all = 0;
 };
 
 // acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales.
@@ -413,7 +419,19 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
             {
                 const u32 tok = ids[q] & 0xFFFFFFu, slot = ids[q] >> 24;
                 const bool ok = (int)slot < g.topk && (int)tok < g.T;       // (a padding group next to a real one: all false)
-                if(ok && !ATOMIC)
+                if(ok && STAGE == 3)
+                {
+                    // the rows are read by whichever workgroup completes the token (gemm_arrive_reduce), possibly on another
+                    // XCD with an L2 of its own: stores at device scope (written through), as the compiler emits them for an
+                    // atomic store of that scope
+                    const u32 orow               = tok * (u32)g.topk + slot;
+                    const unsigned long long dst = (unsigned long long)(out + lane_col) + (unsigned long long)orow * row_bytes;
+                    const v4i d0 = {(int)lo[q][0], (int)hi[q][0], (int)lo[q][1], (int)hi[q][1]};
+                    const v4i d1 = {(int)lo[q][2], (int)hi[q][2], (int)lo[q][3], (int)hi[q][3]};
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\tglobal_store_dwordx4 %0, %2, off offset:16 sc1"
+                                 ::"v"(dst), "v"(d0), "v"(d1) : "memory");
+                }
+                if(ok && !ATOMIC && STAGE != 3)
                 {
                     // (plain stores: marked non-temporal they cost the down GEMM 5 % and the reduction, which then finds
                     // nothing of out3 in the last-level cache, another 4 %)
@@ -437,6 +455,99 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, int e, int nt, 
             __builtin_amdgcn_sched_barrier(0);      // a pair of row groups at a time: keeps the temporaries few
         });
     }
+}
+
+// Stage 3: the top-k reduction inside the down GEMM, by the last arriver.  g.arrive[token, weight tile] starts at the
+// number of the token's slots that take part in the layer (moe_pair_is_kept; written by moe_arrive_init_kernel).  When a
+// tile's rows have been stored to out3 (device-scope stores, waited for by every wave, then a workgroup barrier), the
+// workgroup takes one off the counter of every real row; the workgroup that takes the last one sums the token's
+// slots for these 256 channels from out3 in slot order in fp32 and writes the layer output: the arithmetic of
+// moe_topk_reduce_kernel<.., true>, so the result is the same bit for bit and does not depend on who arrives when.
+// Nobody waits for anybody.  The counter is a device-scope atomic (it orders the arrivals: whoever reads 1 knows that
+// all other slots' stores were complete before their owners decremented), and the rows are read with device-scope
+// loads, because the slots of a token come from up to topk different XCDs whose L2s are not coherent with each other.
+// lds: at least (1 + rows) words that nobody else touches until the function returns (it ends with a barrier).
+template <int MT>
+__device__ __forceinline__ void gemm_arrive_reduce(const GemmArgs& g, int nt, const u32* meta, int ma, u32* lds)
+{
+    const int tid = threadIdx.x;
+    if(tid == 0)
+        lds[0] = 0;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this wave's stores of the tile are complete
+    __syncthreads();                                     // ... and so are the other waves'
+    for(int row = tid; row < ma * 16; row += GEMM_THREADS)
+    {
+        const u32 id  = meta[row];
+        const u32 tok = id & 0xFFFFFFu, slot = id >> 24;
+        if((int)slot < g.topk && (int)tok < g.T)
+        {
+            const int old = __hip_atomic_fetch_sub(g.arrive + (size_t)tok * g.n_tiles + nt, 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            if(old == 1)
+                lds[1 + atomicAdd(&lds[0], 1u)] = tok;
+        }
+    }
+    __syncthreads();
+    const int n = (int)lds[0];
+    // 32 lanes per token, 8 channels (16 bytes) each
+    const int sub = tid & 31;
+    for(int i = tid >> 5; i < n; i += GEMM_THREADS / 32)
+    {
+        const u32 tok = lds[1 + i];
+        const int col = nt * 256 + sub * 8;
+        float acc[8];
+#pragma unroll
+        for(int c = 0; c < 8; c++)
+            acc[c] = 0.f;
+        // NB slots at a time (eight where the tile has registers for it, one in the tiles that run two or more workgroups
+        // per CU on 128 registers): their loads go out together and are waited for once.  The loads are unconditional
+        // (straight-line code between a load and its wait: nothing for the compiler to copy while the load is in flight); a
+        // slot that is left out is read all the same, from memory that nobody wrote, and replaced by +0.0, which leaves
+        // every sum unchanged, as in the reduction kernel.
+        constexpr int NB = MT > 8 ? 8 : 1;
+        for(int s0 = 0; s0 < g.topk; s0 += NB)
+        {
+            v4i v[NB];
+            bool on[NB];
+            unsigned long long src[NB];
+#pragma unroll
+            for(int j = 0; j < NB; j++)
+            {
+                const int sl = s0 + j < g.topk ? s0 + j : g.topk - 1;
+                on[j]  = s0 + j < g.topk && moe_pair_is_kept(g.topk_ids[(size_t)tok * g.topk + sl], g.experts_all, g.expert_mask);
+                src[j] = (unsigned long long)((const uint16_t*)g.out + ((size_t)tok * g.topk + sl) * g.N + col);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for(int j = 0; j < NB; j++)
+                asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v[j]) : "v"(src[j]) : "memory");
+            if constexpr(NB == 8)
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]),
+                             "+v"(v[6]), "+v"(v[7])::"memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0])::"memory");
+#pragma unroll
+            for(int j = 0; j < NB; j++)
+#pragma unroll
+                for(int c = 0; c < 4; c++)
+                {
+                    const u32 w = on[j] ? (u32)v[j][c] : 0u;
+                    acc[2 * c]     += __builtin_bit_cast(float, w << 16);
+                    acc[2 * c + 1] += __builtin_bit_cast(float, w & 0xFFFF0000u);
+                }
+        }
+        if(g.final_f32)
+        {
+            float4* dst = (float4*)((float*)g.final_out + (size_t)tok * g.N + col);
+            dst[0]      = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            dst[1]      = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+        else
+            *(uint4*)((uint16_t*)g.final_out + (size_t)tok * g.N + col) =
+                make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
+                           pack_bf16x2(acc[6], acc[7]));
+    }
+    __syncthreads();                                     // the list is somebody's buffer again from here on
 }
 
 // compute units of the current device (asked once per device, then remembered)

@@ -27,7 +27,9 @@
 #define SCHED_E_MAX 704
 #define SCHED_E_MAX_16 512
 
-// STAGE 1 = gate_up, 2 = down.  MT = row groups of 16 per tile.
+// STAGE 1 = gate_up, 2 = down, 3 = down with the top-k reduction done by the workgroup that stores a token's last
+// slot (gemm_arrive_reduce in gemm_device.h; an option that was built to be measured against stage 2 + the reduction
+// kernel, not what the layer call uses).  MT = row groups of 16 per tile.
 //
 // The kernel is one flat software pipeline over (tile, K-group) pairs: while the MFMAs of K-group ks of a
 // tile run, the activation DMA of K-group ks+1 and the weight loads of K-steps 4(ks+1)..4(ks+1)+3 are in
@@ -327,8 +329,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // is uniform (stage 2: row groups 2, 3 sit 32 rows further in the same descriptor) goes into the scalar offset,
     // which the hardware does not range-check: it stays inside the rows the descriptor covers
     const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1
-    const int w_half     = (STAGE == 2) ? 32 * Kb : 0;
-    const int ws_half    = (STAGE == 2) ? (g.SC / 8) * 256 : 0;
+    const int w_half     = (STAGE >= 2) ? 32 * Kb : 0;
+    const int ws_half    = (STAGE >= 2) ? (g.SC / 8) * 256 : 0;
     auto load_wtile = [&](auto U, auto J, int kt) __attribute__((always_inline)) {
         constexpr int u = decltype(U)::value, j = decltype(J)::value;
         vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
@@ -340,11 +342,14 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // accumulators and epilogue: gemm_device.h
     v4f xacc[TALL ? MT - ACC_SPILL_MT0 : 1];      // the accumulator tiles beyond the accumulation registers (288-row tile)
     auto zero_acc = [&]() __attribute__((always_inline)) { gemm_zero_acc<MT>(xacc); };
-    auto epilogue = [&](const TileId& t, const u32* meta, int ma_t) __attribute__((always_inline)) {
+    // free_lds: the LDS stage that the tile's last K-group has just finished reading (stage 3 keeps a list there)
+    auto epilogue = [&](const TileId& t, const u32* meta, int ma_t, uint8_t* free_lds) __attribute__((always_inline)) {
         if(g.bias)
             gemm_epilogue<STAGE, MT, ACT, ATOMIC, true>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
         else
             gemm_epilogue<STAGE, MT, ACT, ATOMIC, false>(g, t.e, t.nt, t.m_blk * BM, wave, meta, MPAD, ma_t, r, kb, xacc);
+        if constexpr(STAGE == 3)
+            gemm_arrive_reduce<MT>(g, t.nt, meta, ma_t, (u32*)free_lds);
     };
 
     // ---------------------------------------------------------------- pipeline
@@ -540,7 +545,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             // the last MFMAs were issued from assembly: give their results the documented distance to the
             // first VALU read
             asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-            epilogue(cur, lds_meta[mb], ma);
+            epilogue(cur, lds_meta[mb], ma, stage[p]);
             if(!nxt.valid)
                 return false;
             cur = nxt;
@@ -640,12 +645,23 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
             PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel (atomic)");
             return PYHIP_OK;
         }
-    switch(block_m)
+    if constexpr(STAGE == 3)
     {
-        GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(160, 10) GEMM_CASE(192, 12)
-        GEMM_CASE(256, 16) GEMM_CASE(288, 18)
-    default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,160,192,256,288}", block_m); return PYHIP_ERR_INVALID;
+        // built for the tile heights that matter for the comparison with stage 2 + reduction kernel: decode, the
+        // two-workgroup prefill tile and the 288-row tile
+        switch(block_m)
+        {
+            GEMM_CASE(16, 1) GEMM_CASE(128, 8) GEMM_CASE(288, 18)
+        default: pyhip_set_error("moe_gemm2 (reducing): block_m=%d not in {16,128,288}", block_m); return PYHIP_ERR_INVALID;
+        }
     }
+    else
+        switch(block_m)
+        {
+            GEMM_CASE(16, 1) GEMM_CASE(32, 2) GEMM_CASE(64, 4) GEMM_CASE(128, 8) GEMM_CASE(160, 10) GEMM_CASE(192, 12)
+            GEMM_CASE(256, 16) GEMM_CASE(288, 18)
+        default: pyhip_set_error("moe_gemm: block_m=%d not in {16,32,64,128,160,192,256,288}", block_m); return PYHIP_ERR_INVALID;
+        }
 #undef GEMM_CASE
 #undef GEMM_LAUNCH
     PYHIP_CHECK_LAUNCH("moe_gemm_mxfp4_kernel");
@@ -812,4 +828,79 @@ extern "C" int pyhip_moe_gemm2_mxfp4_atomic(const uint8_t* a2_q, const uint8_t* 
     g.SC = (inter / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
     return launch_gemm<2>(g, block_m, 0, stream, true);
+}
+
+// Set-up of the reducing down GEMM (stage 3): arrive[token, weight tile] = the number of the token's slots that take part
+// in the layer; a token without any (all its pairs dropped, or past the local token count) is nobody's to complete: its
+// output row is written here, as zeros.  One wave per token.
+__global__ void __launch_bounds__(256) moe_arrive_init_kernel(const int* topk_ids, const int* expert_mask,
+                                                              const int* num_local_tok, int* arrive, void* out, int out_f32,
+                                                              int T, int topk, int experts, int n_tiles)
+{
+    const int tok = blockIdx.x * 4 + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if(tok >= T)
+        return;
+    int T_local = T;
+    if(num_local_tok)
+    {
+        const int lim = *num_local_tok;
+        T_local       = lim < 0 ? 0 : (lim < T ? lim : T);
+    }
+    int kept = 0;
+    if(tok < T_local)
+        for(int s = 0; s < topk; s++)
+            kept += moe_pair_is_kept(topk_ids[(size_t)tok * topk + s], experts, expert_mask) ? 1 : 0;
+    for(int i = lane; i < n_tiles; i += WAVE)
+        arrive[(size_t)tok * n_tiles + i] = kept;
+    if(kept == 0)
+    {
+        const int words = n_tiles * 256 / (out_f32 ? 1 : 2);
+        u32* row        = (u32*)out + (size_t)tok * words;
+        for(int i = lane; i < words; i += WAVE)
+            row[i] = 0u;
+    }
+}
+
+// The down GEMM that also does the top-k reduction: out3 is written as by pyhip_moe_gemm2_mxfp4, and the workgroup that
+// stores the last of a token's slots for a 256-channel weight tile sums the slots (fp32, slot order, one rounding: the
+// arithmetic of pyhip_moe_topk_reduce_routed, bit for bit) and writes out[tokens, hidden].  No reduction launch and no
+// waiting between workgroups; a deterministic alternative to the reference's atomic epilogue
+// (src/contrib/moe_gemm_mxfp4.py:1334-1398).  arrive: int32 [tokens * hidden / 256] of scratch, initialised here.
+// block_m 16, 128 or 288.  Measured against the two-kernel path, which stays what pyhip_moe_forward uses.
+extern "C" int pyhip_moe_gemm2_mxfp4_reduce(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2,
+                                            const uint8_t* w2_scale, const void* bias2_bf16, const uint32_t* sorted_ids,
+                                            const float* sorted_weights, const uint32_t* sorted_expert_ids,
+                                            const uint32_t* num_valid_ids, const uint32_t* schedule, void* out3_bf16,
+                                            const int32_t* topk_ids, const int32_t* expert_mask,
+                                            const int32_t* num_local_tokens, int32_t* arrive, void* out, int out_is_f32,
+                                            int tokens, int topk, int experts, int hidden, int inter, int block_m,
+                                            int64_t n_blk, hipStream_t stream)
+{
+    int rc = check_common("moe_gemm2_reduce", a2_q, a2_scale, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
+                          out3_bf16, inter, block_m, n_blk, n_blk * block_m);
+    if(rc)
+        return rc;
+    PYHIP_REQUIRE(sorted_weights && topk_ids && arrive && out, "moe_gemm2_reduce: null pointer");
+    PYHIP_REQUIRE(hidden > 0 && hidden % 256 == 0, "moe_gemm2_reduce: hidden=%d must be a multiple of 256", hidden);
+    PYHIP_REQUIRE(tokens > 0 && tokens < (1 << 24) && topk > 0 && topk < 256 && experts > 0, "moe_gemm2_reduce: bad sizes");
+    PYHIP_REQUIRE(((uintptr_t)out3_bf16 % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)arrive % 4) == 0,
+                  "moe_gemm2_reduce: unaligned pointer");
+    hipLaunchKernelGGL(moe_arrive_init_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, topk_ids, expert_mask,
+                       num_local_tokens, arrive, out, out_is_f32, tokens, topk, experts, hidden / 256);
+    PYHIP_CHECK_LAUNCH("moe_arrive_init_kernel");
+    if(n_blk == 0)
+        return PYHIP_OK;
+    GemmArgs g;
+    g.a_q = a2_q; g.a_s = a2_scale; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
+    g.sorted_ids = sorted_ids; g.sorted_w = sorted_weights; g.sorted_e = sorted_expert_ids;
+    g.num_valid = num_valid_ids; g.out = out3_bf16; g.out_q = nullptr; g.out_s = nullptr; g.OSK = 0;
+    g.limit = 0.f;
+    g.sched = schedule; g.E = experts;
+    g.T = tokens; g.topk = topk; g.K = inter; g.N = hidden;
+    g.SK = (inter + 511) / 512 * 16;
+    g.SC = (inter / 32 + 7) / 8 * 8;
+    g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
+    g.arrive = arrive; g.topk_ids = topk_ids; g.expert_mask = expert_mask; g.final_out = out; g.final_f32 = out_is_f32;
+    g.experts_all = experts;
+    return launch_gemm<3>(g, block_m, 0, stream);
 }

@@ -158,6 +158,9 @@ def fused_moe(
     tests/contrib/moe/test_moe.py:76-81); ``topk_reduce="atomic"`` (MXFP4-activation path, row block 16 or 128,
     bf16 output) lets the down GEMM add its results into the output with packed bf16 atomics, the reference's atomic
     variant (src/contrib/moe_gemm_mxfp4.py:1334-1398), instead of the deterministic store + reduction;
+    ``topk_reduce="last_arriver"`` (MXFP4-activation path, row block 16, 128 or 288) keeps the stores and lets the
+    workgroup of the down GEMM that stores a token's last slot sum the slots, in the order and arithmetic of the
+    reduction kernel: the same bits, one launch less;
     ``operand_staging="lds"`` (MXFP4-activation path, 256-row blocks, at most 512 experts) runs both GEMMs on the
     eight-wave tile whose weights, too, are staged through LDS (the tile shape of the reference's prefill kernel,
     src/contrib/moe_gemm_mxfp4.py:318-637) instead of the tiles that load weights straight into registers:
@@ -176,7 +179,7 @@ def fused_moe(
     out_dtype = hidden_states.dtype if dtype is None else dtype
     _require(out_dtype in (torch.bfloat16, torch.float32), "dtype must be bfloat16 or float32", TypeError)
     _require(method in ("auto", "a4w4", "w4a16", "jit", "gluon"), "method=%r" % (method,))
-    _require(topk_reduce in ("store", "atomic"), "topk_reduce=%r" % (topk_reduce,))
+    _require(topk_reduce in ("store", "atomic", "last_arriver"), "topk_reduce=%r" % (topk_reduce,))
     _require(operand_staging in ("registers", "lds"), "operand_staging=%r" % (operand_staging,))
 
     # weights in the plain layout (no ``is_shuffled`` mark) are re-tiled once; the scales always come e8m0-shuffled,
@@ -245,7 +248,12 @@ def fused_moe(
         _require(not w4a16 and bm in (16, 128) and out_dtype == torch.bfloat16,
                  "topk_reduce='atomic' needs the MXFP4-activation path, a row block of 16 or 128 and bf16 output")
 
-    if not return_parts and stage_events is None and not atomic and not lds_tile:
+    arriver = topk_reduce == "last_arriver"
+    if arriver:
+        _require(not w4a16 and bm in (16, 128, 288) and not lds_tile,
+                 "topk_reduce='last_arriver' needs the MXFP4-activation path and a row block of 16, 128 or 288")
+
+    if not return_parts and stage_events is None and not atomic and not lds_tile and not arriver:
         # the whole layer in one library call, intermediates in one workspace: two allocations and one foreign call
         # per layer instead of a dozen of each (the host side is what bounds small layers when they are not replayed
         # from a graph)
@@ -335,6 +343,19 @@ def fused_moe(
                                               _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out),
                                               T, k, global_E, H, I, bm, n_blk, stream)
         _lib.check(rc, "moe_gemm2_mxfp4_atomic")
+        _mark("gemm2", ev)
+    elif arriver:
+        # the down GEMM whose workgroups also sum a token's slots (whoever stores the last one): no reduction launch
+        out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)
+        out = torch.empty(T, H, dtype=out_dtype, device=dev)
+        arrive = torch.empty(T * (H // 256), dtype=torch.int32, device=dev)
+        rc = lib.pyhip_moe_gemm2_mxfp4_reduce(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
+                                              _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
+                                              _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
+                                              _lib.dptr(topk_ids), _lib.dptr(expert_mask), _lib.dptr(num_local_tokens),
+                                              _lib.dptr(arrive), _lib.dptr(out), 1 if out_dtype == torch.float32 else 0,
+                                              T, k, global_E, H, I, bm, n_blk, stream)
+        _lib.check(rc, "moe_gemm2_mxfp4_reduce")
         _mark("gemm2", ev)
     else:
         out3 = torch.empty(T, k, H, dtype=torch.bfloat16, device=dev)

@@ -76,6 +76,8 @@ def test_code_objects_hold_the_kernels():
     gemm = [co.gemm_kernel_name(s, mt, 0, nt).encode() for s in (1, 2) for mt in (1, 2, 4, 8, 10, 12, 16, 18) for nt in (False, True)]
     gemm += [co.gemm_kernel_name(1, mt, 1, nt).encode() for mt in (1, 8, 18) for nt in (False, True)]      # clamped SwiGLU
     gemm += [co.gemm_kernel_name(2, mt, 0, nt, True).encode() for mt in (1, 8) for nt in (False, True)]     # atomic epilogue
+    gemm += [co.gemm_kernel_name(3, mt, 0, nt).encode() for mt in (1, 8, 18) for nt in (False, True)]       # last-arriver reduction
+    gemm += [b"moe_arrive_init_kernel"]
     for name, wanted in (("moe_quant", [b"moe_act_quant_mxfp4_kernel"]),
                          ("moe_reduce", [co.reduce_kernel_name(f, r).encode() for f in (0, 1) for r in (0, 1)]),
                          ("moe_gemm_mxfp4", gemm),

@@ -196,6 +196,22 @@ def test_tile_heights_agree_bit_for_bit(layer):
     assert torch.equal(via_lds, outs[bms[0]])
 
 
+@pytest.mark.parametrize("layer,T,bm", [("dsv3", 8192, 288), ("dsv3", 16, 16), ("qwen3", 8192, 128)], indirect=["layer"])
+def test_last_arriver_reduce_at_full_size(layer, T, bm):
+    """The down GEMM that does the top-k reduction itself (topk_reduce="last_arriver") against the two-kernel path at the
+    benchmark sizes: every token's slots come from up to eight experts' tiles on different XCDs, finished at different
+    times; the output must be the same bit for bit, run after run."""
+    W = layer
+    from pyhip_amd import workloads
+    hidden, tw, ti = workloads.make_inputs(W["shape"], T)
+    print(f"full-size last-arriver case {W['shape']} T={T} block_size_M={bm}", flush=True)
+    want = _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm)
+    for rep in range(3):
+        got = _run(W, hidden, tw, ti, method="a4w4", block_size_M=bm, topk_reduce="last_arriver")
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
+
+
 @pytest.mark.parametrize("layer", ["dsv3"], indirect=True)
 @pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 160, 192, 256)), (5120, (128, 192, 288))])
 def test_load_policies_agree_bit_for_bit(layer, T, bms):

@@ -628,6 +628,48 @@ def test_atomic_topk_reduce_variant(name, T, bm):
     assert metrics.cosine(_f(got), _f(ref32)) >= 0.9999
 
 
+@pytest.mark.parametrize("name,T,bm,bias", [("dsv3_s", 16, 16, False), ("dsv3_s", 200, 16, False), ("tiny", 300, 128, True),
+                                            ("mixtral_s", 700, 288, False), ("odd", 640, 288, True), ("qwen3_s", 257, 128, False)])
+def test_last_arriver_topk_reduce_variant(name, T, bm, bias):
+    """topk_reduce="last_arriver": the down GEMM's workgroups do the top-k reduction themselves, the one that stores a
+    token's last slot for a weight tile sums the slots in slot order.  Same arithmetic as the reduction kernel, so the
+    output must equal the default path's bit for bit, in bf16 and in fp32, whatever the arrival order (three runs), and
+    also where the sort drops pairs (expert mask, local token count): a token all of whose pairs are dropped comes
+    out as zeros."""
+    L = cases.make_layer(name, T, seed=21, bias=bias)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s, block_size_M=bm, method="a4w4", bias1=None if L.bias1 is None else L.bias1.cuda(),
+              bias2=None if L.bias2 is None else L.bias2.cuda())
+    hidden = L.hidden.cuda()
+    print(f"last-arriver case {name} T={T} bm={bm} bias={bias}", flush=True)
+    for dt in (torch.bfloat16, torch.float32):
+        want = fused_moe(hidden, w1, w2, tw, ti, dtype=dt, **kw)
+        for rep in range(3):
+            got, parts = fused_moe(hidden, w1, w2, tw, ti, dtype=dt, topk_reduce="last_arriver", return_parts=True, **kw)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), f"dtype {dt} run {rep}"
+    # out3 is still written in full (callers may want the per-slot results)
+    _, parts0 = fused_moe(hidden, w1, w2, tw, ti, return_parts=True, **kw)
+    assert torch.equal(parts["out3"], parts0["out3"])
+    # dropped pairs: every other expert masked out, and only the first two thirds of the tokens take part
+    E = L.E
+    mask = torch.tensor([e % 2 for e in range(E)], dtype=torch.int32, device="cuda")
+    keep = mask.bool()
+    w1k, w2k = w1[keep].contiguous(), w2[keep].contiguous()
+    w1k.is_shuffled = w2k.is_shuffled = True
+    kwm = dict(kw, w1_scale=w1s.view(E, -1)[keep].contiguous().view(-1, w1s.shape[-1]),
+               w2_scale=w2s.view(E, -1)[keep].contiguous().view(-1, w2s.shape[-1]), expert_mask=mask,
+               num_local_tokens=torch.tensor([max(1, 2 * T // 3)], dtype=torch.int32, device="cuda"),
+               bias1=None if L.bias1 is None else L.bias1.cuda()[keep].contiguous(),
+               bias2=None if L.bias2 is None else L.bias2.cuda()[keep].contiguous())
+    want = fused_moe(hidden, w1k, w2k, tw, ti, **kwm)
+    got = fused_moe(hidden, w1k, w2k, tw, ti, topk_reduce="last_arriver", **kwm)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert (got[max(1, 2 * T // 3):] == 0).all()
+
+
 @pytest.mark.parametrize("T", [2, 3, 7, 31, 63, 128, 200, 255, 256, 768, 2048])
 def test_reference_style_inputs(T):
     """The reference's own accuracy sweep (tests/contrib/moe/test_moe.py:949-1035) draws its inputs differently from
