@@ -21,7 +21,10 @@ reduce) on synthetic inputs that are resident in HBM.  Prints one JSON line.
 
 Measurement modes.  ``--epilogue-comparison``, ``--tile256-comparison TOKENS`` and ``--calibrate-copy MIB`` are not part
 of the default line: each adds one extra object to it (or, for the copy, only extra launches for a counter run) and
-exists so that the command lines quoted in ``profiles/*.txt`` run from this file alone.
+exists so that the command lines quoted in ``profiles/*.txt`` run from this file alone.  ``--frontier`` runs nothing of
+the layer: it times the probe ``pyhip_moe_probe_mfma_stream`` (the 288-row GEMM's inner loop reduced to its MFMA / LDS /
+memory pattern, pyhip_amd/csrc/probe_mfma_stream.hip) and prints one line with what the machine sustains for that
+pattern: matrix-pipeline duty and TB/s per variant.
 """
 import argparse
 import json
@@ -68,6 +71,9 @@ def parse():
                          "256-row tile and the eight-wave 256-row tile with both operands through LDS")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run 3 plain device copies of MIB mebibytes (a yardstick for HBM traffic counters)")
+    ap.add_argument("--frontier", action="store_true",
+                    help="only run the MFMA / HBM-stream probe (six variants of the 288-row GEMM's inner loop) and print "
+                         "matrix-pipeline duty and TB/s of each")
     ap.add_argument("--print-kernel-sources-digest", action="store_true",
                     help="print the digest that profiles/fused_moe_dsv3_hbm_traffic.txt records next to its counters, and exit")
     return ap.parse_args()
@@ -192,6 +198,48 @@ def epilogue_comparison(torch, fused_moe, W, res, block_m, modes=("store", "atom
         acc = {k: sum(v) / len(v) for k, v in acc.items()}
         r[names[mode]] = round(acc["gemm2"] + acc.get("reduce", 0.0), 4)
     return r
+
+
+FRONTIER_VARIANTS = ("mfma_only", "plus_lds_reads", "plus_weight_stream", "plus_lds_dma", "weight_stream_half_the_mfmas",
+                     "weight_stream_no_mfmas")
+
+
+def frontier(torch, iters=4000):
+    """the probe's six variants, one workgroup per CU: ns per MFMA slot (288 slots per wave and iteration), the share of the
+    MFMA-only rate that the matrix pipeline keeps, and the HBM rate of the weight stream (16 KB per wave and iteration)"""
+    import ctypes
+    from pyhip_amd import _lib
+    lib = _lib.load()
+    # random bytes: what the matrix pipeline draws depends on the operands, and real MXFP4 weights look like noise
+    buf = torch.randint(0, 256, ((1 << 30) + (16 << 20),), dtype=torch.uint8, device="cuda",
+                        generator=torch.Generator(device="cuda").manual_seed(0))
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    wgs = ctypes.c_int(0)
+    out, base = {}, None
+    for v, name in enumerate(FRONTIER_VARIANTS):
+        def go(n):
+            _lib.check(lib.pyhip_moe_probe_mfma_stream(v, iters, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), n,
+                                                   ctypes.byref(wgs), _lib.current_stream()), "probe_mfma_stream")
+        # the clock settles under sustained load only: half a second of the same launches first, then 16 timed ones
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.5:
+            go(4)
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        go(16)
+        e1.record()
+        torch.cuda.synchronize()
+        best = e0.elapsed_time(e1) / 16
+        ns_slot = best * 1e6 / (iters * 288.0)
+        base = base or ns_slot
+        mfmas = {4: 0.5, 5: 0.0}.get(v, 1.0)
+        row = {"ms": round(best, 3), "ns_per_mfma_slot": round(ns_slot, 3), "mfma_duty": round(mfmas * base / ns_slot, 4),
+               "pflops": round(mfmas * wgs.value * 4 * 65536 / ns_slot / 1e6, 3)}
+        if v >= 2:
+            row["stream_tbps"] = round(wgs.value * 4 * 16384 * iters / (best * 1e-3) / 1e12, 3)
+        out[name] = row
+    return {"workgroups": wgs.value, "iterations": iters, "variants": out}
 
 
 def tile256_comparison(torch, fused_moe, W, shape, tokens):
@@ -332,6 +380,11 @@ def main():
     a = parse()
     if a.print_kernel_sources_digest:
         print(kernel_sources_digest())
+        return
+    if a.frontier:
+        import torch
+        torch.cuda.set_device(0)
+        print(json.dumps({"mfma_hbm_frontier": frontier(torch)}))
         return
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU only (--gpus %d requested); expert-parallel sharding over "

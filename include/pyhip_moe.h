@@ -253,6 +253,19 @@ int pyhip_moe_topk_reduce_routed(const void* in_bf16, void* out, int64_t tokens,
 int pyhip_moe_zero_fill(void* p, int64_t bytes, pyhip_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Measurement probe (no counterpart in the reference; used by bench.py --frontier only): the inner loop of the 288-row
+ * MXFP4 GEMM reduced to its instruction and memory pattern, one workgroup of four waves per CU, `iters` K-groups of 288
+ * scaled FP4 MFMAs per wave.  variant 0: MFMAs only; 1: + LDS operand reads; 2: + the weight stream (16 KB per wave and
+ * K-group from `buf`, prefetched one K-group ahead); 3: + 29 LDS-DMA operations per K-group; 4: as 2 with every second
+ * MFMA replaced by VALU moves; 5: as 2 with none.  Enqueues `launches` launches on `stream`; the caller times them.
+ *   buf        device buffer of at least 2^30 + 2^24 bytes, read only (fill it with noise: what the matrix pipeline
+ *              draws, and with it the clock, depends on the operands)
+ *   sink       device int32[4], never written in practice
+ *   workgroups receives the workgroups per launch (the CU count) */
+int pyhip_moe_probe_mfma_stream(int variant, int iters, const void* buf, int64_t buf_bytes, int32_t* sink, int launches,
+                                int* workgroups, pyhip_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
  * The whole layer in one call: sort (+ input quantisation) -> gate_up GEMM -> down GEMM -> top-k reduce, i.e. the
  * body of the reference's fused_moe (src/contrib/fused_moe.py:128-576) for the MXFP4 path, with every
  * intermediate buffer carved out of `workspace` (pyhip_moe_forward_workspace_bytes() bytes, 256-byte aligned)

@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libpyhip_moe.so")
-SOURCES = ["capi.hip", "moe_sort.hip", "moe_quant.hip", "moe_gemm_mxfp4.hip", "moe_gemm_mxfp4_wide.hip", "moe_gemm_w4a16.hip", "moe_reduce.hip", "moe_router.hip", "moe_forward.hip", "moe_forward_static.hip"]
+SOURCES = ["capi.hip", "moe_sort.hip", "moe_quant.hip", "moe_gemm_mxfp4.hip", "moe_gemm_mxfp4_wide.hip", "moe_gemm_w4a16.hip", "moe_reduce.hip", "moe_router.hip", "moe_forward.hip", "moe_forward_static.hip", "probe_mfma_stream.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -30,7 +30,7 @@ def _run(cmd):
 
 CO_DIR = os.path.join(HERE, "co")
 # every source that holds kernels is also shipped as a stand-alone code object (see build_co); the rest of SOURCES
-# (capi, moe_forward, moe_forward_static) is host code only
+# (capi, moe_forward, moe_forward_static) is host code only; the measurement probe stays in the library
 CO_SOURCES = ["moe_quant.hip", "moe_reduce.hip", "moe_gemm_mxfp4.hip", "moe_sort.hip", "moe_router.hip",
               "moe_gemm_w4a16.hip", "moe_gemm_mxfp4_wide.hip"]
 

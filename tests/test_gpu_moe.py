@@ -670,6 +670,27 @@ def test_last_arriver_topk_reduce_variant(name, T, bm, bias):
     assert (got[max(1, 2 * T // 3):] == 0).all()
 
 
+def test_mfma_stream_probe_runs():
+    """the measurement probe behind bench.py --frontier: every variant launches, finishes and reports the CU count;
+    bad arguments are refused before anything is launched"""
+    import ctypes
+    from pyhip_amd import _lib
+    lib = _lib.load()
+    buf = torch.zeros((1 << 30) + (16 << 20), dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    wgs = ctypes.c_int(0)
+    for v in range(6):
+        print(f"probe variant {v}", flush=True)
+        _lib.check(lib.pyhip_moe_probe_mfma_stream(v, 20, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), 2, ctypes.byref(wgs),
+                                                   _lib.current_stream()), "probe")
+        torch.cuda.synchronize()
+    assert wgs.value == torch.cuda.get_device_properties(0).multi_processor_count
+    assert (sink == 0).all()
+    assert lib.pyhip_moe_probe_mfma_stream(6, 20, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), 1, None, None) == 1
+    assert lib.pyhip_moe_probe_mfma_stream(2, 20, _lib.dptr(buf), 1 << 30, _lib.dptr(sink), 1, None, None) == 1
+    assert b"buffer" in lib.pyhip_moe_last_error()
+
+
 @pytest.mark.parametrize("T", [2, 3, 7, 31, 63, 128, 200, 255, 256, 768, 2048])
 def test_reference_style_inputs(T):
     """The reference's own accuracy sweep (tests/contrib/moe/test_moe.py:949-1035) draws its inputs differently from
