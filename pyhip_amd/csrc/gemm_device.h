@@ -76,6 +76,48 @@ __device__ __forceinline__ void mfma_one(v4i w, v4i a, int ws, int a_scale, v4f*
                      : [c] "n"(A0), [e] "n"(A0 + 3), [w] "v"(w), [a] "v"(a), [ws] "v"(ws), [as] "v"(a_scale),
                        [wl] "n"(WB & 1), [wh] "n"(WB >> 1), [al] "n"(U & 1), [ah] "n"(U >> 1));
 }
+// The four MFMAs of a row group behind a test of the tile's number of row groups that hold real rows: a row group at or
+// beyond that number is padding (zeros in LDS: its MFMAs add nothing) and is jumped over.  One compare and one branch
+// per row group, so it is only used for the last few row groups of the tall tiles, the ones that are empty often: a
+// tile height is chosen so that an expert's rows usually fit one block, which leaves the block's tail unused more often
+// than not.  (A guard around EVERY row group costs more issue time than the skipped MFMAs save, see above; and what the
+// matrix pipeline does not execute it does not draw power for, which on this part is what the memory stream gets.)
+template <int U, int MTI, int MT>
+__device__ __forceinline__ void mfma_row_group_guarded(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale,
+                                                       int groups_with_rows, v4f* xacc = nullptr)
+{
+    constexpr int A0 = MTI * 4, A1 = (MT + MTI) * 4, A2 = (2 * MT + MTI) * 4, A3 = (3 * MT + MTI) * 4;
+    constexpr int WL = U & 1;                         // weight-scale byte (kt%2)*2 + (row%32)/16: op_sel_hi = kt%2 ...
+    static_assert(A2 + 3 < 256, "only weight row group 3 may overflow the accumulation registers");
+#define PYHIP_MFMA_TXT(ACC, W, WS, LO) \
+    "v_mfma_scale_f32_16x16x128_f8f6f4 " ACC ", " W ", %[a], " ACC ", " WS ", %[as] op_sel:[" LO ",%[al],0] op_sel_hi:[%[wh],%[ah],0] cbsz:4 blgp:4\n\t"
+    if constexpr(acc_in_vgprs<MT, MTI>())
+        asm volatile("s_cmp_le_u32 %[n], %[mti]\n\ts_cbranch_scc1 1f\n\t"
+                     PYHIP_MFMA_TXT("a[%[c0]:%[e0]]", "%[w0]", "%[s01]", "0")
+                     PYHIP_MFMA_TXT("a[%[c1]:%[e1]]", "%[w1]", "%[s01]", "1")
+                     PYHIP_MFMA_TXT("a[%[c2]:%[e2]]", "%[w2]", "%[s23]", "0")
+                     PYHIP_MFMA_TXT("%[xa]", "%[w3]", "%[s23]", "1")
+                     "1:"
+                     : [xa] "+v"(*xacc)
+                     : [n] "s"(groups_with_rows), [mti] "n"(MTI), [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3),
+                       [c2] "n"(A2), [e2] "n"(A2 + 3), [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2), [w3] "v"(w3), [a] "v"(a),
+                       [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [wh] "n"(WL), [al] "n"(U & 1), [ah] "n"(U >> 1)
+                     : "scc");
+    else
+        asm volatile("s_cmp_le_u32 %[n], %[mti]\n\ts_cbranch_scc1 1f\n\t"
+                     PYHIP_MFMA_TXT("a[%[c0]:%[e0]]", "%[w0]", "%[s01]", "0")
+                     PYHIP_MFMA_TXT("a[%[c1]:%[e1]]", "%[w1]", "%[s01]", "1")
+                     PYHIP_MFMA_TXT("a[%[c2]:%[e2]]", "%[w2]", "%[s23]", "0")
+                     PYHIP_MFMA_TXT("a[%[c3]:%[e3]]", "%[w3]", "%[s23]", "1")
+                     "1:"
+                     :
+                     : [n] "s"(groups_with_rows), [mti] "n"(MTI), [c0] "n"(A0), [e0] "n"(A0 + 3), [c1] "n"(A1), [e1] "n"(A1 + 3),
+                       [c2] "n"(A2), [e2] "n"(A2 + 3), [c3] "n"(A3), [e3] "n"(A3 + 3), [w0] "v"(w0), [w1] "v"(w1), [w2] "v"(w2),
+                       [w3] "v"(w3), [a] "v"(a), [s01] "v"(ws01), [s23] "v"(ws23), [as] "v"(a_scale), [wh] "n"(WL), [al] "n"(U & 1),
+                       [ah] "n"(U >> 1)
+                     : "scc");
+#undef PYHIP_MFMA_TXT
+}
 // the four MFMAs of a row group back to back (the eight-wave kernel, whose two waves per SIMD fill each other's gaps)
 template <int U, int MTI, int MT>
 __device__ __forceinline__ void mfma_row_group(v4i w0, v4i w1, v4i w2, v4i w3, v4i a, int ws01, int ws23, int a_scale,

@@ -366,6 +366,8 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     // at 128 rows: gpt-oss shape, 4096 tokens, layer 0.573 against 0.597 ms; Mixtral shape, 512 tokens, 0.216 against
     // 0.224 ms).
     constexpr bool SPREAD = MT > 8;
+    // the last GUARDED row groups of a tall tile are jumped over when they hold no real rows (mfma_row_group_guarded)
+    constexpr int GUARDED = MT == 18 ? 2 : MT > 8 ? 3 : 0;
     using VS = VmSchedule<MA, NPF, SPREAD ? 2 : 1>;
     static_assert(VS::younger(0) <= 63 && VS::younger(1) <= 63 && VS::younger(2) <= 63 && VS::younger(3) <= 63,
                   "the vector-memory counter has six bits");
@@ -508,6 +510,23 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
                 // weight-scale byte = (kt%2)*2 + (row%32)/16 ; activation-scale byte = kt%4
                 if constexpr(!SPREAD && n + RA < 4 * MA)
                     lds_read(std::integral_constant<int, n + RA>{});
+                if constexpr(SPREAD && mt >= MT - GUARDED)
+                {
+                    // one of the tile's last row groups, which are padding more often than not: everything else that
+                    // belongs to the row group first (same order as always: the waits count on it), then its four MFMAs
+                    // behind one test of the tile's number of row groups with real rows
+                    if constexpr(n + RA < 4 * MA)
+                        lds_read(std::integral_constant<int, n + RA>{});
+                    static_for<4>([&](auto G) __attribute__((always_inline)) { issue_gap(N{}, G, TS{}, kpre); });
+                    __builtin_amdgcn_sched_barrier(0);
+                    v4f* xa = nullptr;
+                    if constexpr(acc_in_vgprs<MT, mt>())
+                        xa = &xacc[mt - ACC_SPILL_MT0];
+                    mfma_row_group_guarded<u, mt, MT>(wf[u][0], wf[u][1], wf[u][2], wf[u][3], af, w_sc[p][u >> 1],
+                                                      w_sc[p][2 + (u >> 1)], asc, ma, xa);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                else
                 static_for<4>([&](auto J) __attribute__((always_inline)) {
                     constexpr int j = decltype(J)::value;
                     v4f* xa = nullptr;
