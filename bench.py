@@ -201,7 +201,8 @@ def epilogue_comparison(torch, fused_moe, W, res, block_m, modes=("store", "atom
 
 
 FRONTIER_VARIANTS = ("mfma_only", "plus_lds_reads", "plus_weight_stream", "plus_lds_dma", "weight_stream_half_the_mfmas",
-                     "weight_stream_no_mfmas")
+                     "weight_stream_no_mfmas", "all_with_weights_from_l2",
+                     "rows128_mfma_plus_lds_reads", "rows128_all_with_weights_from_l2", "rows128_all_with_weight_stream")
 
 
 def frontier(torch, iters=4000):
@@ -231,13 +232,17 @@ def frontier(torch, iters=4000):
         e1.record()
         torch.cuda.synchronize()
         best = e0.elapsed_time(e1) / 16
-        ns_slot = best * 1e6 / (iters * 288.0)
+        # MFMA slots per wave and iteration: 288 (288-row tile), 128 (128-row tile, two waves per SIMD)
+        slots = 128.0 if v >= 7 else 288.0
+        ns_slot = best * 1e6 / (iters * slots) / (2 if v >= 7 else 1)       # per SIMD
         base = base or ns_slot
         mfmas = {4: 0.5, 5: 0.0}.get(v, 1.0)
         row = {"ms": round(best, 3), "ns_per_mfma_slot": round(ns_slot, 3), "mfma_duty": round(mfmas * base / ns_slot, 4),
-               "pflops": round(mfmas * wgs.value * 4 * 65536 / ns_slot / 1e6, 3)}
-        if v >= 2:
+               "pflops": round(mfmas * wgs.value * 4 * slots * iters * 65536 / (best * 1e-3) / 1e15, 3)}
+        if v in (2, 3, 4, 5, 9):
             row["stream_tbps"] = round(wgs.value * 4 * 16384 * iters / (best * 1e-3) / 1e12, 3)
+        if v in (6, 8):
+            row["l2_weight_tbps"] = round(wgs.value * 4 * 16384 * iters / (best * 1e-3) / 1e12, 3)
         out[name] = row
     return {"workgroups": wgs.value, "iterations": iters, "variants": out}
 

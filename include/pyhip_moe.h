@@ -257,11 +257,13 @@ int pyhip_moe_zero_fill(void* p, int64_t bytes, pyhip_stream_t stream);
  * MXFP4 GEMM reduced to its instruction and memory pattern, one workgroup of four waves per CU, `iters` K-groups of 288
  * scaled FP4 MFMAs per wave.  variant 0: MFMAs only; 1: + LDS operand reads; 2: + the weight stream (16 KB per wave and
  * K-group from `buf`, prefetched one K-group ahead); 3: + 29 LDS-DMA operations per K-group; 4: as 2 with every second
- * MFMA replaced by VALU moves; 5: as 2 with none.  Enqueues `launches` launches on `stream`; the caller times them.
+ * MFMA replaced by VALU moves; 5: as 2 with none; 6: as 3 with the weight tiles from an L2-resident region; 7, 8, 9: the
+ * 128-row tile's pattern (two workgroups per CU, 128 MFMAs per wave and K-group): MFMAs + operand reads; everything with
+ * weights from the L2; everything with weights streamed.  Enqueues `launches` launches on `stream`; the caller times them.
  *   buf        device buffer of at least 2^30 + 2^24 bytes, read only (fill it with noise: what the matrix pipeline
  *              draws, and with it the clock, depends on the operands)
  *   sink       device int32[4], never written in practice
- *   workgroups receives the workgroups per launch (the CU count) */
+ *   workgroups receives the workgroups per launch (the CU count, or twice that) */
 int pyhip_moe_probe_mfma_stream(int variant, int iters, const void* buf, int64_t buf_bytes, int32_t* sink, int launches,
                                 int* workgroups, pyhip_stream_t stream);
 

@@ -13,30 +13,39 @@
 //           3  + the LDS-DMA operations
 //           4  as 2, every second MFMA replaced by four VALU moves (the same issue time, half the matrix work)
 //           5  as 2, every MFMA replaced: the load stream alone at the MFMA loop's pace
+//           6  as 3, the weight tiles from a region that stays in the L2 (the compute-bound case: few experts, many rows)
+//   and the same for the 128-row tile's pattern (two workgroups per CU, 128 MFMAs, 32 operand reads, 16 weight tiles
+//   and 10 LDS-DMA operations per wave and K-group):
+//           7  MFMAs + LDS operand reads          8  + LDS-DMA + weight tiles from the L2          9  + ... streamed from HBM
 #include "gemm_device.h"
 
-#define PROBE_LDS_BYTES (96 * 1024)             // more than half a CU's LDS: one workgroup per CU
+#define PROBE_LDS_BYTES(RG) ((RG) == 18 ? 96 * 1024 : 64 * 1024)     // one workgroup per CU, or two
 #define PROBE_STREAM_MASK 0x3FFFFFFF            // the stream wraps inside the first GiB of the buffer
 #define PROBE_MIN_BYTES ((1ll << 30) + (16ll << 20))
 
-template <int V>
-__global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int iters, const uint8_t* buf, int* sink)
+// V: what takes part (0..5 above); RG: row groups per K-step (18: the 288-row tile, 8: the 128-row tile); CACHED: the weight
+// tiles come from 16 KB per wave that are read again and again (L2 hits) instead of a stream through the first GiB
+template <int V, int RG, bool CACHED>
+__global__ void __launch_bounds__(GEMM_THREADS, (RG == 18 ? 1 : 2)) probe_mfma_stream_kernel(int iters, const uint8_t* buf, int* sink)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     asm volatile("" ::: "a0", "a63");               // the 16 accumulator tiles the MFMAs below name
-    __shared__ __attribute__((aligned(16))) uint8_t lds[PROBE_LDS_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[PROBE_LDS_BYTES(RG)];
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-    for(int i = tid; i < PROBE_LDS_BYTES / 4; i += GEMM_THREADS)
+    for(int i = tid; i < PROBE_LDS_BYTES(RG) / 4; i += GEMM_THREADS)
         ((u32*)lds)[i] = (u32)i * 2654435761u;
     __syncthreads();
     constexpr bool LDS_READS = V >= 1, STREAM = V >= 2, DMA = V == 3;
+    static_assert(!CACHED || V == 3, "the cached source exists for the full pattern only");
     constexpr int MFMA_EVERY = V == 4 ? 2 : V == 5 ? 0 : 1;     // 1: every slot an MFMA; 2: every second; 0: none
-    // stream: wave w of workgroup b reads 4 KB pieces at piece index (4 b + w) of consecutive 4 MiB chunks; the chunk
+    // stream: wave w of workgroup b reads 4 KB pieces at piece index (4 b + w) of consecutive 8 MiB chunks; the chunk
     // offset goes into the scalar offset (not range-checked: the mask keeps it inside the first GiB)
     const v4i rs      = make_rsrc(buf, 0x7FFFFFF0u);
-    const int gw      = (int)((blockIdx.x * 4 + wave) & 1023);
-    const int v_strm  = lane * 16 + gw * 4096;
+    const int gw      = (int)((blockIdx.x * 4 + wave) & 2047);
+    const int v_strm  = lane * 16 + gw * (CACHED ? 16384 : 4096);
+    constexpr int NDMA = RG == 18 ? 29 : 10, DMA_RGS = RG == 18 ? 2 * RG : RG;   // LDS-DMA operations and the row groups they are spread over
+    constexpr int WSTEP = RG / 4;                               // row groups between two weight tiles of a K-step
     const int v_dma   = lane * 16 + gw * 4096;                  // 4 KB per wave, read again every iteration: cache hits
     const u32 lds_dma = (u32)__builtin_amdgcn_readfirstlane((int)lds_addr_of(lds + 32768 + wave * 4096));
     const uint8_t* rd = lds + lane * 16;
@@ -54,7 +63,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
     const int sc = 0x7f7f7f7f;                                  // scale bytes 127: 2^0
     gemm_zero_acc<4>();
     auto slot = [&](auto NN, auto JJ) __attribute__((always_inline)) {
-        constexpr int n = decltype(NN)::value, j = decltype(JJ)::value, u = n / 18;
+        constexpr int n = decltype(NN)::value, j = decltype(JJ)::value, u = n / RG;
         constexpr int k = n * 4 + j;
         if constexpr(MFMA_EVERY == 1 || (MFMA_EVERY == 2 && k % 2 == 0))
             mfma_one<u, n % 4, 4, j>(wf[u * 4 + j], LDS_READS ? af[n % 3] : wf[0], sc, sc);
@@ -69,7 +78,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
         constexpr int i = decltype(II)::value;
         vm_load_b128<(i % 4) * 1024, false>(wf[i], v_strm, rs, sx);
         if constexpr(i % 4 == 3)
-            sx = (sx + 0x400000) & PROBE_STREAM_MASK;
+            sx = CACHED ? (sx + 4096) & 0x3FFF : (sx + 0x800000) & PROBE_STREAM_MASK;
     };
     if constexpr(LDS_READS)
     {
@@ -78,7 +87,7 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
     }
     for(int it = 0; it < iters; it++)
     {
-        static_for<72>([&](auto NN) __attribute__((always_inline)) {
+        static_for<4 * RG>([&](auto NN) __attribute__((always_inline)) {
             constexpr int n = decltype(NN)::value;
             __builtin_amdgcn_sched_barrier(0);
             static_for<4>([&](auto JJ) __attribute__((always_inline)) {
@@ -87,17 +96,18 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr(LDS_READS && j == 0)
                     af[(n + 2) % 3] = *(const v4i*)(rd + ((n + 2) % 16) * 1024);
-                // 29 LDS-DMA operations over the first two K-steps (row groups 0..35), as the GEMM spreads them
-                if constexpr(DMA && j >= 1 && n < 36)
+                // the LDS-DMA operations over the first two K-steps (288-row tile) or the first (128-row tile), as the GEMM
+                // spreads them
+                if constexpr(DMA && j >= 1 && n < DMA_RGS)
                 {
-                    constexpr int s = n * 3 + j - 1;                    // slot 0..107
-                    if constexpr((s * 29) / 108 != ((s + 1) * 29) / 108)
-                        vm_dma_b128<((s * 29 / 108) % 4) * 1024, 0>(v_dma, rs, 0, lds_dma);
+                    constexpr int s = n * 3 + j - 1, NS = DMA_RGS * 3;  // slot 0 .. NS-1
+                    if constexpr((s * NDMA) / NS != ((s + 1) * NDMA) / NS)
+                        vm_dma_b128<((s * NDMA / NS) % 4) * 1024, 0>(v_dma, rs, 0, lds_dma);
                 }
                 // the weight tiles of K-step u go out during K-step u + 1 (u = 3: after the last row group)
-                constexpr int m  = n >= 18 ? n - 18 : 0;               // row groups since the start of K-step 1
-                constexpr int ti = (m / 18) * 4 + (m % 18) / 4 % 4;    // tile u * 4 + j goes out at row group 18 (u + 1) + 4 j
-                if constexpr(STREAM && j == 3 && n >= 18 && m % 18 % 4 == 0 && m % 18 / 4 < 4)
+                constexpr int m  = n >= RG ? n - RG : 0;               // row groups since the start of K-step 1
+                constexpr int ti = (m / RG) * 4 + (m % RG) / WSTEP % 4;   // tile u * 4 + j goes out at row group RG (u + 1) + WSTEP j
+                if constexpr(STREAM && j == 3 && n >= RG && m % RG % WSTEP == 0 && m % RG / WSTEP < 4)
                     stream_load(std::integral_constant<int, ti>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -107,7 +117,10 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
             static_for<4>([&](auto JJ) __attribute__((always_inline)) { stream_load(std::integral_constant<int, 12 + decltype(JJ)::value>{}); });
             // everything but this iteration's youngest 12 weight tiles has landed (the DMA operations, the tiles of
             // K-step 0, and all of the previous iteration's): the GEMM's wait at the end of a K-group
-            asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+            if constexpr(RG == 18)
+                asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // (128-row tile: all its weight tiles follow the LDS-DMA)
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -127,25 +140,33 @@ __global__ void __launch_bounds__(GEMM_THREADS, 1) probe_mfma_stream_kernel(int 
 extern "C" int pyhip_moe_probe_mfma_stream(int variant, int iters, const void* buf, int64_t buf_bytes, int32_t* sink,
                                        int launches, int* workgroups, hipStream_t stream)
 {
-    PYHIP_REQUIRE(variant >= 0 && variant <= 5, "probe_mfma_stream: variant=%d not in 0..5", variant);
+    PYHIP_REQUIRE(variant >= 0 && variant <= 9, "probe_mfma_stream: variant=%d not in 0..9", variant);
     PYHIP_REQUIRE(iters > 0 && launches > 0, "probe_mfma_stream: bad counts");
     PYHIP_REQUIRE(buf && sink && buf_bytes >= PROBE_MIN_BYTES && ((uintptr_t)buf % 16) == 0,
                   "probe_mfma_stream: needs an aligned buffer of at least %lld bytes", (long long)PROBE_MIN_BYTES);
     const int cus = device_cu_count();
+    const int wgs = variant >= 7 ? 2 * cus : cus;
     if(workgroups)
-        *workgroups = cus;
+        *workgroups = wgs;
+#define PROBE_LAUNCH(V, RG, C) \
+    hipLaunchKernelGGL((probe_mfma_stream_kernel<V, RG, C>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink)
     for(int l = 0; l < launches; l++)
     {
         switch(variant)
         {
-        case 0: hipLaunchKernelGGL(probe_mfma_stream_kernel<0>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
-        case 1: hipLaunchKernelGGL(probe_mfma_stream_kernel<1>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
-        case 2: hipLaunchKernelGGL(probe_mfma_stream_kernel<2>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
-        case 3: hipLaunchKernelGGL(probe_mfma_stream_kernel<3>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
-        case 4: hipLaunchKernelGGL(probe_mfma_stream_kernel<4>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
-        default: hipLaunchKernelGGL(probe_mfma_stream_kernel<5>, dim3(cus), dim3(GEMM_THREADS), 0, stream, iters, (const uint8_t*)buf, sink); break;
+        case 0: PROBE_LAUNCH(0, 18, false); break;
+        case 1: PROBE_LAUNCH(1, 18, false); break;
+        case 2: PROBE_LAUNCH(2, 18, false); break;
+        case 3: PROBE_LAUNCH(3, 18, false); break;
+        case 4: PROBE_LAUNCH(4, 18, false); break;
+        case 5: PROBE_LAUNCH(5, 18, false); break;
+        case 6: PROBE_LAUNCH(3, 18, true); break;
+        case 7: PROBE_LAUNCH(1, 8, false); break;
+        case 8: PROBE_LAUNCH(3, 8, true); break;
+        default: PROBE_LAUNCH(3, 8, false); break;
         }
     }
+#undef PROBE_LAUNCH
     PYHIP_CHECK_LAUNCH("probe_mfma_stream_kernel");
     return PYHIP_OK;
 }

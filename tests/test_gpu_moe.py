@@ -679,14 +679,14 @@ def test_mfma_stream_probe_runs():
     buf = torch.zeros((1 << 30) + (16 << 20), dtype=torch.uint8, device="cuda")
     sink = torch.zeros(4, dtype=torch.int32, device="cuda")
     wgs = ctypes.c_int(0)
-    for v in range(6):
+    for v in range(10):
         print(f"probe variant {v}", flush=True)
         _lib.check(lib.pyhip_moe_probe_mfma_stream(v, 20, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), 2, ctypes.byref(wgs),
                                                    _lib.current_stream()), "probe")
         torch.cuda.synchronize()
-    assert wgs.value == torch.cuda.get_device_properties(0).multi_processor_count
+    assert wgs.value == 2 * torch.cuda.get_device_properties(0).multi_processor_count     # (the last variants: two per CU)
     assert (sink == 0).all()
-    assert lib.pyhip_moe_probe_mfma_stream(6, 20, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), 1, None, None) == 1
+    assert lib.pyhip_moe_probe_mfma_stream(10, 20, _lib.dptr(buf), buf.numel(), _lib.dptr(sink), 1, None, None) == 1
     assert lib.pyhip_moe_probe_mfma_stream(2, 20, _lib.dptr(buf), 1 << 30, _lib.dptr(sink), 1, None, None) == 1
     assert b"buffer" in lib.pyhip_moe_last_error()
 
