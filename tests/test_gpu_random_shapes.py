@@ -80,3 +80,36 @@ def test_random_shape(seed):
         e16 = np.abs(got16 - ref16).max() / rms16
         print(f"  w4a16 vs oracle: max|err|/rms={e16:.3e} cosine={metrics.cosine(got16, ref16):.8f}", flush=True)
         assert metrics.cosine(got16, ref16) >= TOL_COS and metrics.calc_diff(got16, ref16) <= 0.01 and e16 <= 5e-2
+
+
+@pytest.mark.parametrize("method,T", [("a4w4", 700), ("a4w4", 33), ("w4a16", 20)])
+def test_extreme_routings(method, T):
+    """Routings at the edges of what the sort sees: every token on the same expert(s) (one expert with all the rows and
+    many row blocks, the others with none), and a token naming the same expert in two of its slots (two pairs, two rows
+    of that expert, as the reference's sorter counts them)."""
+    L = cases.make_layer("tiny", T, seed=41)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    hidden = L.hidden.cuda()
+    kw = dict(w1_scale=w1s, w2_scale=w2s, dtype=torch.float32, method=method)
+    g = np.random.default_rng(42)
+    for name in ("one_expert", "two_experts", "duplicates"):
+        if name == "one_expert":
+            ids = np.full((T, L.k), 5, np.int32)
+            ids[:, 1] = 2                                    # slot 0 on expert 5, slot 1 on expert 2, for every token
+        elif name == "two_experts":
+            ids = np.stack([np.full(T, 7, np.int32), g.integers(0, 2, T).astype(np.int32) * 3], axis=1)
+        else:
+            ids = L.topk_ids.copy()
+            ids[::3, 1] = ids[::3, 0]                        # every third token: the same expert twice
+        tw = g.random((T, L.k), dtype=np.float32) + 0.1
+        print(f"extreme-routing case {name} T={T} method={method}", flush=True)
+        out = fused_moe(hidden, w1, w2, torch.from_numpy(tw).cuda(), torch.from_numpy(ids).cuda(), **kw)
+        torch.cuda.synchronize()
+        ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, tw, ids, act="a4" if method == "a4w4" else "a16")
+        got = _f(out)
+        rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+        err, cos = metrics.max_err_over_rms(got, ref), metrics.cosine(got, ref)
+        frac = float((np.abs(got - ref) > TOL_MAX * rms).mean())
+        print(f"  vs oracle: max|err|/rms={err:.3e} cosine={cos:.8f} beyond-bound fraction={frac:.2e}", flush=True)
+        assert np.isfinite(got).all() and cos >= TOL_COS and metrics.calc_diff(got, ref) <= 0.01
+        assert (frac <= 2e-3 and err <= 0.1) if method == "a4w4" else err <= 5e-2
