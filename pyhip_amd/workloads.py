@@ -1,5 +1,5 @@
-"""Synthetic MoE layers of the benchmark shapes, generated on the device (torch), and the routers
-that produce ``topk_weight`` / ``topk_ids``.  Used by ``bench.py`` and the large-size GPU tests.
+"""Synthetic MoE layers of the benchmark shapes (weights generated on the device, inputs and routing on the CPU) and
+the routers that produce ``topk_weight`` / ``topk_ids``.  Used by ``bench.py`` and the large-size GPU tests.
 
 Shapes (experts, top-k, hidden, intermediate):
   tiny 8/2/1024/512, Mixtral-8x7B 8/2/4096/14336, gpt-oss-120b 128/4/2880/2880 (+biases),
@@ -89,12 +89,14 @@ def make_weights(shape, device="cuda", seed=0, experts_per_chunk=8):
 
 
 def make_inputs(shape, tokens, device="cuda", seed=1):
+    """hidden states and routing of a call, drawn with a CPU generator and routed on the CPU, so that any machine
+    reproduces them bit for bit (the weights, gigabytes of them, are drawn on the device: see make_weights)"""
     cfg = SHAPES[shape] if isinstance(shape, str) else shape
-    g = torch.Generator(device=device).manual_seed(seed)
-    hidden = torch.randn(tokens, cfg["H"], generator=g, device=device).to(torch.bfloat16)
-    logits = torch.randn(tokens, cfg["E"], generator=g, device=device)
+    g = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(tokens, cfg["H"], generator=g).to(torch.bfloat16)
+    logits = torch.randn(tokens, cfg["E"], generator=g)
     topk_w, topk_ids = route(cfg, logits)
-    return hidden, topk_w, topk_ids
+    return hidden.to(device), topk_w.to(device), topk_ids.to(device)
 
 
 def algorithmic_work(shape, tokens, topk_ids):
