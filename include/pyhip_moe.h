@@ -131,14 +131,20 @@ int pyhip_moe_act_quant_mxfp4(const void* x_bf16, int64_t row_stride_elems, int6
  *                afterwards, and it replaces the second aiter.get_hip_quant + moe_mxfp4_sort call of
  *                tests/contrib/moe/test_moe.py:732-744.  Needs inter % 512 == 0.  At least one of a2 and
  *                a2_q must be given.
+ *   hidden_pad, inter_pad   how many of the last columns of `hidden` / of the last rows of each half of `inter` are
+ *                zero padding (the reference operator's hidden_pad / intermediate_pad, src/contrib/fused_moe.py:149-150:
+ *                shapes such as gpt-oss's 2880 arrive padded to the tiles' multiples).  0 <= pad < size.  The padding of
+ *                the weights must be zeros; the kernels do not fetch groups of 32 (stage 2: 64) weight rows that are all
+ *                padding, nor (16- and 32-row blocks) groups of 32 columns that are; results are the same as with 0, 0.
  * block_m must equal the block_size the sort ran with and `experts` the expert count it ran with;
  * block_m is 16, 32, 64, 128, 160, 192, 256 or 288; hidden % 512 == 0, inter % 128 == 0.  schedule: as written by pyhip_moe_sorting, or NULL (then one
  * workgroup per tile and worst-case block is launched, as the reference does). */
 int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                           const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
                           const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q,
-                          uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                          int64_t n_blk, int activation, float swiglu_limit, pyhip_stream_t stream);
+                          uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int hidden_pad,
+                          int inter_pad, int block_m, int64_t n_blk, int activation, float swiglu_limit,
+                          pyhip_stream_t stream);
 
 /* Stage 2: down grouped GEMM, times the routing weight.  Replaces moe_gemm_mxfp4(gate_up=False),
  * src/contrib/moe_gemm_mxfp4.py:1291-1333 (launch: tests/contrib/moe/test_moe.py:751-763).
@@ -150,12 +156,13 @@ int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale, const uint
  *                  count) keep whatever the buffer held.  Reduce with pyhip_moe_topk_reduce_routed, which leaves
  *                  those slots out by the same rule, or clear out3 first when the plain pyhip_moe_topk_reduce is
  *                  used with a routing that drops pairs.
+ *   hidden_pad, inter_pad   as for stage 1: here the last hidden_pad rows of w2 and its last inter_pad columns
  * inter % 512 == 0, hidden % 256 == 0. */
 int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
                           const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
                           const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
                           const uint32_t* schedule, void* out3_bf16, int tokens, int topk, int experts, int hidden,
-                          int inter, int block_m, int64_t n_blk, pyhip_stream_t stream);
+                          int inter, int hidden_pad, int inter_pad, int block_m, int64_t n_blk, pyhip_stream_t stream);
 
 /* The same two GEMMs on the eight-wave tile of 256 rows x 256 weight rows whose operands BOTH go through LDS (LDS-DMA
  * into a ring of five weight stages and three activation stages, two wave rows half a K-step apart), the tile shape of
@@ -276,6 +283,8 @@ int pyhip_moe_probe_mfma_stream(int variant, int iters, const void* buf, int64_t
  *   w1, w2, scales, biases, expert_mask, num_local_tokens: as for the step-by-step entry points above
  *   out           bf16 (or fp32 when out_is_f32 != 0) [tokens, hidden]
  *   experts       the expert count the router saw (the length of expert_mask when one is given)
+ *   hidden, inter the sizes the weights have, padding included; hidden_pad, inter_pad: how much of them is zero padding
+ *                 (as for pyhip_moe_gemm1_mxfp4; the bf16-activation kernels take no notice)
  *   block_m       the row block: 16/32/64, with MXFP4 activations also 128/160/192/256/288
  *   w4a16         0 = MXFP4 activations (pyhip_moe_gemm*_mxfp4), 1 = bf16 activations (pyhip_moe_gemm*_w4a16)
  * pyhip_moe_pick_block_m / pyhip_moe_pick_w4a16 give the choices the reference's operator makes inside fused_moe
@@ -289,8 +298,8 @@ int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_stride, const 
                       const uint8_t* w2, const uint8_t* w2_scale, const void* bias1_bf16, const void* bias2_bf16,
                       const int32_t* topk_ids, const float* topk_weights, const int32_t* expert_mask,
                       const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk, int experts,
-                      int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
-                      void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
+                      int hidden, int inter, int hidden_pad, int inter_pad, int block_m, int w4a16, int split_k,
+                      int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes, pyhip_stream_t stream);
 
 /* pyhip_moe_forward with the router inside the call: gating f32 [tokens, experts] in (n_group / topk_group /
  * renormalize as for pyhip_moe_route_sorting), the picks out in topk_ids / topk_weights next to the layer output.
@@ -300,9 +309,9 @@ int pyhip_moe_forward_routed(const void* hidden_bf16, int64_t hidden_row_stride,
                              const void* bias1_bf16, const void* bias2_bf16, const float* gating, int n_group,
                              int topk_group, int renormalize, int32_t* topk_ids, float* topk_weights,
                              const int32_t* expert_mask, const int32_t* num_local_tokens, void* out, int out_is_f32,
-                             int tokens, int topk, int experts, int hidden, int inter, int block_m, int w4a16,
-                             int split_k, int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
-                             pyhip_stream_t stream);
+                             int tokens, int topk, int experts, int hidden, int inter, int hidden_pad, int inter_pad,
+                             int block_m, int w4a16, int split_k, int activation, float swiglu_limit, void* workspace,
+                             int64_t workspace_bytes, pyhip_stream_t stream);
 
 /* pyhip_moe_forward without the workspace argument: the intermediates live in a device array that belongs to the
  * library (64 MiB, pyhip_moe_forward_static_capacity(); one copy per GPU, held until the process ends).  It has no
@@ -321,8 +330,8 @@ int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_row_stride,
                              const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
                              const float* topk_weights, const int32_t* expert_mask, const int32_t* num_local_tokens,
                              void* out, int out_is_f32, int tokens, int topk, int experts, int hidden, int inter,
-                             int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
-                             pyhip_stream_t stream);
+                             int hidden_pad, int inter_pad, int block_m, int w4a16, int split_k, int activation,
+                             float swiglu_limit, pyhip_stream_t stream);
 
 #ifdef __cplusplus
 }

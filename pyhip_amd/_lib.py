@@ -25,20 +25,20 @@ SIGNATURES = {
     "pyhip_moe_pick_w4a16": (_I, [_L, _I, _I, _I]),
     "pyhip_moe_zero_fill": (_I, [_P, _L, _P]),
     "pyhip_moe_forward_workspace_bytes": (_L, [_L, _I, _I, _I, _I, _I, _I]),
-    "pyhip_moe_forward": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
+    "pyhip_moe_forward": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                _I, _F, _P, _L, _P]),
     "pyhip_moe_route_sorting": (_I, [_P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _L, _I,
                                      _P, _P, _P]),
     "pyhip_moe_forward_routed": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I,
-                                      _I, _I, _I, _I, _I, _I, _F, _P, _L, _P]),
+                                      _I, _I, _I, _I, _I, _I, _I, _I, _F, _P, _L, _P]),
     "pyhip_moe_forward_static_capacity": (_L, []),
-    "pyhip_moe_forward_static": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I,
+    "pyhip_moe_forward_static": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                       _I, _F, _P]),
     "pyhip_moe_sorting_quant": (_I, [_P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _L, _L, _I, _P, _P, _P]),
     "pyhip_moe_act_scale_stride": (_L, [_I]),
     "pyhip_moe_act_quant_mxfp4": (_I, [_P, _L, _L, _I, _P, _P, _P, _P]),
-    "pyhip_moe_gemm1_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _F, _P]),
-    "pyhip_moe_gemm2_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
+    "pyhip_moe_gemm1_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _I, _F, _P]),
+    "pyhip_moe_gemm2_mxfp4": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _P]),
     "pyhip_moe_gemm1_mxfp4_lds": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _F, _P]),
     "pyhip_moe_gemm2_mxfp4_lds": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _P]),
     "pyhip_moe_gemm2_mxfp4_atomic": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _P]),

@@ -24,7 +24,9 @@ class GemmArgs(ctypes.Structure):
                 ("n_blk", _I), ("n_tiles", _I), ("a_rows", _I), ("E", _I),
                 # STAGE 3 (down GEMM with the last-arriver reduction) only
                 ("arrive", _P), ("topk_ids", _P), ("expert_mask", _P), ("final_out", _P), ("final_f32", _I),
-                ("experts_all", _I)]
+                ("experts_all", _I),
+                # zero padding at the end of the weight matrices: rows (per half in stage 1) and columns left unfetched
+                ("n_pad", _I), ("k_pad", _I)]
 
 
 class QuantArgs(ctypes.Structure):

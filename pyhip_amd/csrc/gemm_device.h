@@ -32,6 +32,11 @@ struct GemmArgs
     const int* expert_mask = nullptr;   // ... and the expert mask ([experts_all] or null), for the drop rule
     void* final_out        = nullptr;   // [T, N] bf16, or fp32 when final_f32 != 0
     int final_f32 = 0, experts_all = 0;
+    // zero padding at the end of the weight matrices (shapes that are not multiples of the tiles arrive padded): the last
+    // n_pad rows of every expert's weight matrix (stage 1: of its gate half and of its up half) and the last k_pad
+    // columns are zeros.  Waves whose weight rows are all padding fetch nothing (the registers then hold the zeros that
+    // an out-of-range fetch returns: the same product), and so do, in the 16- and 32-row tiles, lanes past the real columns.
+    int n_pad = 0, k_pad = 0;
 };
 
 // acc += W(16 rows x 128 K, e2m1) * A(128 K x 16 rows, e2m1) with per-lane e8m0 block scales.

@@ -16,10 +16,10 @@ int pyhip_moe_sorting_quant(const int32_t*, const float*, int, int, int, int, co
                             uint8_t*, uint8_t*, hipStream_t);
 int pyhip_moe_gemm1_mxfp4(const uint8_t*, const uint8_t*, const uint8_t*, const uint8_t*, const void*, const uint32_t*,
                           const uint32_t*, const uint32_t*, const uint32_t*, void*, uint8_t*, uint8_t*, int, int, int, int,
-                          int, int, int64_t, int, float, hipStream_t);
+                          int, int, int, int, int64_t, int, float, hipStream_t);
 int pyhip_moe_gemm2_mxfp4(const uint8_t*, const uint8_t*, const uint8_t*, const uint8_t*, const void*, const uint32_t*,
                           const float*, const uint32_t*, const uint32_t*, const uint32_t*, void*, int, int, int, int, int,
-                          int, int64_t, hipStream_t);
+                          int, int, int, int64_t, hipStream_t);
 int pyhip_moe_gemm1_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const uint32_t*,
                           const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, int, float, hipStream_t);
 int pyhip_moe_gemm2_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const float*,
@@ -178,8 +178,8 @@ static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, cons
                         const uint8_t* w2, const uint8_t* w2_scale, const void* bias1_bf16, const void* bias2_bf16,
                         const Router& router, int32_t* topk_ids, float* topk_weights, const int32_t* expert_mask,
                         const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk, int experts,
-                        int hidden, int inter, int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
-                        void* workspace, int64_t workspace_bytes, hipStream_t stream)
+                        int hidden, int inter, int hidden_pad, int inter_pad, int block_m, int w4a16, int split_k,
+                        int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes, hipStream_t stream)
 {
     PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && w2 && w2_scale && topk_ids && topk_weights && out,
                   "moe_forward: null pointer");
@@ -228,12 +228,12 @@ static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, cons
     else
     {
         rc = pyhip_moe_gemm1_mxfp4(ws + l.a1_q, ws + l.a1_s, w1, w1_scale, bias1_bf16, s_ids, s_e, n_valid, sched, nullptr,
-                                   ws + l.a2_q, ws + l.a2_s, tokens, topk, experts, hidden, inter, block_m, l.n_blk,
-                                   activation, swiglu_limit, stream);
+                                   ws + l.a2_q, ws + l.a2_s, tokens, topk, experts, hidden, inter, hidden_pad, inter_pad,
+                                   block_m, l.n_blk, activation, swiglu_limit, stream);
         if(rc)
             return rc;
         rc = pyhip_moe_gemm2_mxfp4(ws + l.a2_q, ws + l.a2_s, w2, w2_scale, bias2_bf16, s_ids, s_w, s_e, n_valid, sched,
-                                   out3, tokens, topk, experts, hidden, inter, block_m, l.n_blk, stream);
+                                   out3, tokens, topk, experts, hidden, inter, hidden_pad, inter_pad, block_m, l.n_blk, stream);
     }
     if(rc)
         return rc;
@@ -249,14 +249,14 @@ extern "C" int pyhip_moe_forward(const void* hidden_bf16, int64_t hidden_row_str
                                  const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
                                  const float* topk_weights, const int32_t* expert_mask,
                                  const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens, int topk,
-                                 int experts, int hidden, int inter, int block_m, int w4a16, int split_k,
-                                 int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
-                                 hipStream_t stream)
+                                 int experts, int hidden, int inter, int hidden_pad, int inter_pad, int block_m,
+                                 int w4a16, int split_k, int activation, float swiglu_limit, void* workspace,
+                                 int64_t workspace_bytes, hipStream_t stream)
 {
     return forward_impl(hidden_bf16, hidden_row_stride, w1, w1_scale, w2, w2_scale, bias1_bf16, bias2_bf16, Router{},
                         const_cast<int32_t*>(topk_ids), const_cast<float*>(topk_weights), expert_mask, num_local_tokens,
-                        out, out_is_f32, tokens, topk, experts, hidden, inter, block_m, w4a16, split_k, activation,
-                        swiglu_limit, workspace, workspace_bytes, stream);
+                        out, out_is_f32, tokens, topk, experts, hidden, inter, hidden_pad, inter_pad, block_m, w4a16,
+                        split_k, activation, swiglu_limit, workspace, workspace_bytes, stream);
 }
 
 // The layer with its router: gating scores in, and the picks (topk_ids, topk_weights) out next to the layer output.
@@ -267,13 +267,15 @@ extern "C" int pyhip_moe_forward_routed(const void* hidden_bf16, int64_t hidden_
                                         int topk_group, int renormalize, int32_t* topk_ids, float* topk_weights,
                                         const int32_t* expert_mask, const int32_t* num_local_tokens, void* out,
                                         int out_is_f32, int tokens, int topk, int experts, int hidden, int inter,
-                                        int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
-                                        void* workspace, int64_t workspace_bytes, hipStream_t stream)
+                                        int hidden_pad, int inter_pad, int block_m, int w4a16, int split_k,
+                                        int activation, float swiglu_limit, void* workspace, int64_t workspace_bytes,
+                                        hipStream_t stream)
 {
     PYHIP_REQUIRE(gating, "moe_forward_routed: null gating scores");
     Router r;
     r.gating = gating; r.n_group = n_group; r.topk_group = topk_group; r.renormalize = renormalize;
     return forward_impl(hidden_bf16, hidden_row_stride, w1, w1_scale, w2, w2_scale, bias1_bf16, bias2_bf16, r, topk_ids,
                         topk_weights, expert_mask, num_local_tokens, out, out_is_f32, tokens, topk, experts, hidden, inter,
-                        block_m, w4a16, split_k, activation, swiglu_limit, workspace, workspace_bytes, stream);
+                        hidden_pad, inter_pad, block_m, w4a16, split_k, activation, swiglu_limit, workspace, workspace_bytes,
+                        stream);
 }

@@ -8,7 +8,7 @@ int64_t pyhip_moe_forward_workspace_bytes(int64_t tokens, int topk, int experts,
                                           int w4a16);
 int pyhip_moe_forward(const void*, int64_t, const uint8_t*, const uint8_t*, const uint8_t*, const uint8_t*, const void*,
                       const void*, const int32_t*, const float*, const int32_t*, const int32_t*, void*, int, int, int, int,
-                      int, int, int, int, int, int, float, void*, int64_t, hipStream_t);
+                      int, int, int, int, int, int, int, int, float, void*, int64_t, hipStream_t);
 }
 
 // The same layer for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -64,8 +64,9 @@ extern "C" int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_
                                         const void* bias1_bf16, const void* bias2_bf16, const int32_t* topk_ids,
                                         const float* topk_weights, const int32_t* expert_mask,
                                         const int32_t* num_local_tokens, void* out, int out_is_f32, int tokens,
-                                        int topk, int experts, int hidden, int inter, int block_m, int w4a16,
-                                        int split_k, int activation, float swiglu_limit, hipStream_t stream)
+                                        int topk, int experts, int hidden, int inter, int hidden_pad, int inter_pad,
+                                        int block_m, int w4a16, int split_k, int activation, float swiglu_limit,
+                                        hipStream_t stream)
 {
     PYHIP_REQUIRE(tokens > 0 && topk > 0 && experts > 0 && hidden > 0 && inter > 0 && block_m > 0,
                   "moe_forward_static: bad sizes");
@@ -80,6 +81,6 @@ extern "C" int pyhip_moe_forward_static(const void* hidden_bf16, int64_t hidden_
         return rc;
     return pyhip_moe_forward(hidden_bf16, hidden_row_stride, w1, w1_scale, w2, w2_scale, bias1_bf16, bias2_bf16, topk_ids,
                              topk_weights, expert_mask, num_local_tokens, out, out_is_f32, tokens, topk, experts, hidden,
-                             inter, block_m, w4a16, split_k, activation, swiglu_limit, ws, PYHIP_STATIC_SCRATCH_BYTES,
-                             stream);
+                             inter, hidden_pad, inter_pad, block_m, w4a16, split_k, activation, swiglu_limit, ws,
+                             PYHIP_STATIC_SCRATCH_BYTES, stream);
 }

@@ -274,15 +274,17 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
             for(int h = 0; h < 2; h++)
             {
                 const size_t row = (size_t)t.e * g.N + h * I + t.nt * 128 + wave * 32;
-                wrs[h]           = make_rsrc(g.w + row * Kb, (u32)(32 * Kb));
-                wsrs[h]          = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)sc_tile);
+                const bool real  = t.nt * 128 + wave * 32 < I - g.n_pad;       // (rows of padding: nothing to fetch)
+                wrs[h]           = make_rsrc(g.w + row * Kb, real ? (u32)(32 * Kb) : 0u);
+                wsrs[h]          = make_rsrc(g.w_s + (row / 32) * sc_tile, real ? (u32)sc_tile : 0u);
             }
         }
         else
         {
             const size_t row = (size_t)t.e * g.N + t.nt * 256 + wave * 64;
-            wrs[0] = wrs[1] = make_rsrc(g.w + row * Kb, (u32)(64 * Kb));
-            wsrs[0] = wsrs[1] = make_rsrc(g.w_s + (row / 32) * sc_tile, (u32)(2 * sc_tile));
+            const bool real  = t.nt * 256 + wave * 64 < g.N - g.n_pad;
+            wrs[0] = wrs[1] = make_rsrc(g.w + row * Kb, real ? (u32)(64 * Kb) : 0u);
+            wsrs[0] = wsrs[1] = make_rsrc(g.w_s + (row / 32) * sc_tile, real ? (u32)(2 * sc_tile) : 0u);
         }
         // (all the reads first, from a clamped position and without a branch between them: one LDS round trip instead of
         // one per slot)
@@ -331,9 +333,18 @@ __global__ void __launch_bounds__(GEMM_THREADS, (MT > 8 ? 1 : 2)) moe_gemm_mxfp4
     const int w_voff[2]  = {lane * 16, lane * 16 + 16 * Kb};                    // row groups j = 2h, 2h+1
     const int w_half     = (STAGE >= 2) ? 32 * Kb : 0;
     const int ws_half    = (STAGE >= 2) ? (g.SC / 8) * 256 : 0;
+    // The 16- and 32-row tiles are bound by the weight stream: there, lanes whose 32 columns of a K-step are all padding
+    // fetch nothing (their offset is pushed out of the descriptor's range; the register gets the zeros the padding holds).
+    const int k_real = g.K - g.k_pad;
     auto load_wtile = [&](auto U, auto J, int kt) __attribute__((always_inline)) {
         constexpr int u = decltype(U)::value, j = decltype(J)::value;
-        vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
+        if constexpr(MT <= 2)
+        {
+            const int away = kt * 128 + kb * 32 >= k_real ? (int)0x80000000u : 0;
+            vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1] + away, wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
+        }
+        else
+            vm_load_b128<0, NT>(wf[u][j], w_voff[j & 1], wrs[j >> 1], kt * 1024 + (j >> 1) * w_half);
     };
     auto load_wtiles = [&](auto U, int kt) __attribute__((always_inline)) {
         static_for<4>([&](auto J) __attribute__((always_inline)) { load_wtile(U, J, kt); });
@@ -708,9 +719,13 @@ static int check_common(const char* name, const void* a_q, const void* a_s, cons
 static int gemm1_impl(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t* w1, const uint8_t* w1_scale,
                       const void* bias1_bf16, const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids,
                       const uint32_t* num_valid_ids, const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q,
-                      uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                      int64_t n_blk, int activation, float swiglu_limit, hipStream_t stream, bool lds)
+                      uint8_t* a2_scale, int tokens, int topk, int experts, int hidden, int inter, int hidden_pad,
+                      int inter_pad, int block_m, int64_t n_blk, int activation, float swiglu_limit, hipStream_t stream,
+                      bool lds)
 {
+    PYHIP_REQUIRE(hidden_pad >= 0 && hidden_pad < hidden && inter_pad >= 0 && inter_pad < inter,
+                  "moe_gemm1: hidden_pad=%d / inter_pad=%d outside [0, hidden=%d) / [0, inter=%d)", hidden_pad, inter_pad,
+                  hidden, inter);
     PYHIP_REQUIRE(a2_bf16 || a2_q, "moe_gemm1: no output buffer");
     PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
                   "moe_gemm1: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
@@ -735,6 +750,7 @@ static int gemm1_impl(const uint8_t* a_q, const uint8_t* a_scale, const uint8_t*
     g.SK = (hidden + 511) / 512 * 16;
     g.SC = (hidden / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = inter / 128; g.a_rows = tokens;
+    g.n_pad = inter_pad; g.k_pad = hidden_pad;
     return launch_gemm<1>(g, block_m, activation, stream, false, lds);
 }
 
@@ -742,12 +758,13 @@ extern "C" int pyhip_moe_gemm1_mxfp4(const uint8_t* a_q, const uint8_t* a_scale,
                                      const uint8_t* w1_scale, const void* bias1_bf16, const uint32_t* sorted_ids,
                                      const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,
                                      const uint32_t* schedule, void* a2_bf16, uint8_t* a2_q, uint8_t* a2_scale,
-                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, int activation, float swiglu_limit, hipStream_t stream)
+                                     int tokens, int topk, int experts, int hidden, int inter, int hidden_pad,
+                                     int inter_pad, int block_m, int64_t n_blk, int activation, float swiglu_limit,
+                                     hipStream_t stream)
 {
     return gemm1_impl(a_q, a_scale, w1, w1_scale, bias1_bf16, sorted_ids, sorted_expert_ids, num_valid_ids, schedule,
-                      a2_bf16, a2_q, a2_scale, tokens, topk, experts, hidden, inter, block_m, n_blk, activation,
-                      swiglu_limit, stream, false);
+                      a2_bf16, a2_q, a2_scale, tokens, topk, experts, hidden, inter, hidden_pad, inter_pad, block_m, n_blk,
+                      activation, swiglu_limit, stream, false);
 }
 
 // The gate_up GEMM on the eight-wave 256-row tile whose operands both go through LDS (moe_gemm_mxfp4_wide.hip); the
@@ -760,16 +777,19 @@ extern "C" int pyhip_moe_gemm1_mxfp4_lds(const uint8_t* a_q, const uint8_t* a_sc
                                          int activation, float swiglu_limit, hipStream_t stream)
 {
     return gemm1_impl(a_q, a_scale, w1, w1_scale, bias1_bf16, sorted_ids, sorted_expert_ids, num_valid_ids, schedule,
-                      a2_bf16, a2_q, a2_scale, tokens, topk, experts, hidden, inter, 256, n_blk, activation, swiglu_limit,
-                      stream, true);
+                      a2_bf16, a2_q, a2_scale, tokens, topk, experts, hidden, inter, 0, 0, 256, n_blk, activation,
+                      swiglu_limit, stream, true);
 }
 
 static int gemm2_impl(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_t* w2, const uint8_t* w2_scale,
                       const void* bias2_bf16, const uint32_t* sorted_ids, const float* sorted_weights,
                       const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids, const uint32_t* schedule,
-                      void* out3_bf16, int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                      int64_t n_blk, hipStream_t stream, bool lds)
+                      void* out3_bf16, int tokens, int topk, int experts, int hidden, int inter, int hidden_pad,
+                      int inter_pad, int block_m, int64_t n_blk, hipStream_t stream, bool lds)
 {
+    PYHIP_REQUIRE(hidden_pad >= 0 && hidden_pad < hidden && inter_pad >= 0 && inter_pad < inter,
+                  "moe_gemm2: hidden_pad=%d / inter_pad=%d outside [0, hidden=%d) / [0, inter=%d)", hidden_pad, inter_pad,
+                  hidden, inter);
     int rc = check_common("moe_gemm2", a2_q, a2_scale, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                           out3_bf16, inter, block_m, n_blk, n_blk * block_m);
     if(rc)
@@ -789,6 +809,7 @@ static int gemm2_impl(const uint8_t* a2_q, const uint8_t* a2_scale, const uint8_
     g.SK = (inter + 511) / 512 * 16;
     g.SC = (inter / 32 + 7) / 8 * 8;
     g.n_blk = (int)n_blk; g.n_tiles = hidden / 256; g.a_rows = (int)(n_blk * block_m);
+    g.n_pad = hidden_pad; g.k_pad = inter_pad;
     return launch_gemm<2>(g, block_m, 0, stream, false, lds);
 }
 
@@ -796,11 +817,12 @@ extern "C" int pyhip_moe_gemm2_mxfp4(const uint8_t* a2_q, const uint8_t* a2_scal
                                      const uint8_t* w2_scale, const void* bias2_bf16, const uint32_t* sorted_ids,
                                      const float* sorted_weights, const uint32_t* sorted_expert_ids,
                                      const uint32_t* num_valid_ids, const uint32_t* schedule, void* out3_bf16,
-                                     int tokens, int topk, int experts, int hidden, int inter, int block_m,
-                                     int64_t n_blk, hipStream_t stream)
+                                     int tokens, int topk, int experts, int hidden, int inter, int hidden_pad,
+                                     int inter_pad, int block_m, int64_t n_blk, hipStream_t stream)
 {
     return gemm2_impl(a2_q, a2_scale, w2, w2_scale, bias2_bf16, sorted_ids, sorted_weights, sorted_expert_ids,
-                      num_valid_ids, schedule, out3_bf16, tokens, topk, experts, hidden, inter, block_m, n_blk, stream, false);
+                      num_valid_ids, schedule, out3_bf16, tokens, topk, experts, hidden, inter, hidden_pad, inter_pad, block_m,
+                      n_blk, stream, false);
 }
 
 // the down GEMM on the same tile
@@ -812,7 +834,7 @@ extern "C" int pyhip_moe_gemm2_mxfp4_lds(const uint8_t* a2_q, const uint8_t* a2_
                                          hipStream_t stream)
 {
     return gemm2_impl(a2_q, a2_scale, w2, w2_scale, bias2_bf16, sorted_ids, sorted_weights, sorted_expert_ids,
-                      num_valid_ids, schedule, out3_bf16, tokens, topk, experts, hidden, inter, 256, n_blk, stream, true);
+                      num_valid_ids, schedule, out3_bf16, tokens, topk, experts, hidden, inter, 0, 0, 256, n_blk, stream, true);
 }
 
 // The down GEMM with the top-k reduction in its epilogue: every (token, slot) result is added into out[token, :]

@@ -189,7 +189,7 @@ def fused_moe(
     # hidden_pad / intermediate_pad: the weights arrive zero-padded to the kernels' tile multiples and the last
     # hidden_pad (intermediate_pad) channels are padding.  The activations may come at the padded width (the
     # reference's convention) or at the true width, in which case they are widened here and the result is
-    # returned at the true width.
+    # returned at the true width.  The MXFP4-activation GEMMs are told the pads and leave the weights' padding unfetched.
     _require(0 <= hidden_pad < w1u.shape[2] * 2 and 0 <= intermediate_pad < w1u.shape[1] // 2, "bad hidden_pad / intermediate_pad")
     narrow = hidden_pad > 0 and hidden_states.shape[1] == w1u.shape[2] * 2 - hidden_pad
     if narrow:
@@ -267,9 +267,9 @@ def fused_moe(
         rc = lib.pyhip_moe_forward(_lib.dptr(x), x.stride(0), _lib.dptr(w1u), _lib.dptr(w1s), _lib.dptr(w2u),
                                    _lib.dptr(w2s), _lib.dptr(bias1), _lib.dptr(bias2), _lib.dptr(topk_ids),
                                    _lib.dptr(topk_weight), _lib.dptr(expert_mask), _lib.dptr(num_local_tokens),
-                                   _lib.dptr(out), 1 if out_dtype == torch.float32 else 0, T, k, global_E, H, I, bm,
-                                   1 if w4a16 else 0, splitk, act, limit, _lib.dptr(ws), ws_bytes,
-                                   _lib.current_stream())
+                                   _lib.dptr(out), 1 if out_dtype == torch.float32 else 0, T, k, global_E, H, I,
+                                   hidden_pad, intermediate_pad, bm, 1 if w4a16 else 0, splitk, act, limit,
+                                   _lib.dptr(ws), ws_bytes, _lib.current_stream())
         _lib.check(rc, "moe_forward")
         return out[:, : H - hidden_pad] if narrow else out
 
@@ -331,7 +331,8 @@ def fused_moe(
         rc = lib.pyhip_moe_gemm1_mxfp4(_lib.dptr(a1_q), _lib.dptr(a1_s), _lib.dptr(w1u), _lib.dptr(w1s),
                                        _lib.dptr(bias1), _lib.dptr(sorted_ids), _lib.dptr(sorted_e),
                                        _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(a2), _lib.dptr(a2_q),
-                                       _lib.dptr(a2_s), T, k, global_E, H, I, bm, n_blk, act, limit, stream)
+                                       _lib.dptr(a2_s), T, k, global_E, H, I, hidden_pad, intermediate_pad, bm, n_blk,
+                                       act, limit, stream)
     _lib.check(rc, "moe_gemm1_mxfp4")
     ev = _mark("gemm1", ev)
     if atomic:
@@ -368,7 +369,7 @@ def fused_moe(
             rc = lib.pyhip_moe_gemm2_mxfp4(_lib.dptr(a2_q), _lib.dptr(a2_s), _lib.dptr(w2u), _lib.dptr(w2s),
                                            _lib.dptr(bias2), _lib.dptr(sorted_ids), _lib.dptr(sorted_w),
                                            _lib.dptr(sorted_e), _lib.dptr(num_valid), _lib.dptr(sched), _lib.dptr(out3),
-                                           T, k, global_E, H, I, bm, n_blk, stream)
+                                           T, k, global_E, H, I, hidden_pad, intermediate_pad, bm, n_blk, stream)
         _lib.check(rc, "moe_gemm2_mxfp4")
         ev = _mark("gemm2", ev)
         out = torch.empty(T, H, dtype=out_dtype, device=dev)
@@ -387,11 +388,12 @@ def fused_moe(
 def fused_moe_routed(hidden_states, w1, w2, gating_output, topk, renormalize=True, num_expert_group=0, topk_group=0,
                      w1_scale=None, w2_scale=None, expert_mask=None, activation=ActivationType.Silu,
                      block_size_M=None, num_local_tokens=None, dtype=None, bias1=None, bias2=None, splitk=0,
-                     method="auto", swiglu_limit=None, return_routing=False):
+                     method="auto", swiglu_limit=None, return_routing=False, hidden_pad=0, intermediate_pad=0):
     """``fused_topk`` (or ``grouped_topk`` when ``num_expert_group > 0``) followed by ``fused_moe``, as the reference's
     callers chain them (tests/contrib/moe/test_fused_moe.py:38-60), in one library call: for up to 64 tokens the
     router runs inside the sort's launch.  ``gating_output`` f32 [T, E], E a multiple of 64 (use ``fused_topk`` +
-    ``fused_moe`` otherwise).  -> out, or (out, topk_weights, topk_ids) with ``return_routing``."""
+    ``fused_moe`` otherwise).  ``hidden_pad`` / ``intermediate_pad`` as for ``fused_moe``, with the activations at the
+    padded width.  -> out, or (out, topk_weights, topk_ids) with ``return_routing``."""
     lib = _lib.load()
     _require(activation in (ActivationType.Silu, ActivationType.Swiglu), "SiLU- or SwiGLU-gated experts only")
     act = 1 if activation == ActivationType.Swiglu else 0
@@ -434,7 +436,8 @@ def fused_moe_routed(hidden_states, w1, w2, gating_output, topk, renormalize=Tru
                                       _lib.dptr(w2s), _lib.dptr(bias1), _lib.dptr(bias2), _lib.dptr(g),
                                       int(num_expert_group), int(topk_group), 1 if renormalize else 0, _lib.dptr(ti),
                                       _lib.dptr(tw), _lib.dptr(expert_mask), _lib.dptr(num_local_tokens), _lib.dptr(out),
-                                      1 if out_dtype == torch.float32 else 0, T, topk, global_E, H, I, bm,
-                                      1 if w4a16 else 0, splitk, act, limit, _lib.dptr(ws), ws_bytes, _lib.current_stream())
+                                      1 if out_dtype == torch.float32 else 0, T, topk, global_E, H, I, int(hidden_pad),
+                                      int(intermediate_pad), bm, 1 if w4a16 else 0, splitk, act, limit, _lib.dptr(ws),
+                                      ws_bytes, _lib.current_stream())
     _lib.check(rc, "moe_forward_routed")
     return (out, tw, ti) if return_routing else out

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.pyhip_moe_abi_version() == 7
+    assert lib.pyhip_moe_abi_version() == 8
 
 
 def test_size_helpers():
@@ -53,10 +53,15 @@ def test_argument_errors_are_reported():
     rc = lib.pyhip_moe_sorting_quant(one, one, 4, 2, 8, 16, None, None, one, one, one, one, None, one, 256,
                                      None, 1024, 4, 1024, one, one, None)
     assert rc == 1 and b"null pointer" in lib.pyhip_moe_last_error()
-    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1000, 512, 16, 4, 0, 0.0, None)
+    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1000, 512, 0, 0, 16, 4, 0, 0.0, None)
     assert rc == 1 and b"multiple of 512" in lib.pyhip_moe_last_error()
-    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 48, 4, None)
+    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 0, 0, 48, 4, None)
     assert rc == 1 and b"block_m" in lib.pyhip_moe_last_error()
+    # pads are a part of the size they pad
+    rc = lib.pyhip_moe_gemm1_mxfp4(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1024, 512, 1024, 0, 16, 4, 0, 0.0, None)
+    assert rc == 1 and b"hidden_pad" in lib.pyhip_moe_last_error()
+    rc = lib.pyhip_moe_gemm2_mxfp4(one, one, one, one, None, one, one, one, one, None, one, 4, 2, 8, 1024, 512, 0, -1, 16, 4, None)
+    assert rc == 1 and b"inter_pad" in lib.pyhip_moe_last_error()
     # the tile with both operands through LDS only exists with the sort's schedule
     rc = lib.pyhip_moe_gemm1_mxfp4_lds(one, one, one, one, None, one, one, one, None, one, None, None, 4, 2, 8, 1024, 1024, 4, 0, 0.0, None)
     assert rc == 1 and b"schedule missing" in lib.pyhip_moe_last_error()

@@ -239,6 +239,36 @@ def test_padded_shape_matches_oracle(T, bm, bias):
     _end_to_end(_f(out_narrow), ref, ref_a2, nflip1)
 
 
+@pytest.mark.parametrize("T,bm", [(24, 16), (90, 32), (150, 64), (300, 128), (500, 288)])
+def test_padding_is_left_unfetched_and_changes_nothing(T, bm):
+    """hidden 1376 and inter 1312 padded to 1536: the last K-step of 128 columns is all padding in both GEMMs, and so are
+    whole waves' weight rows.  Told the pads, the GEMMs leave that part of the weights unfetched (the 16- and 32-row tiles
+    also the K-step); the padding being zeros, the result must equal, bit for bit, the one computed with the padded
+    sizes passed off as real ones (pads 0, everything fetched), in the one-call path and step by step, and must match
+    the oracle on the unpadded problem."""
+    L = cases.make_layer("gptoss_s", T, seed=5, bias=True, H=1376, I=1312)
+    w1, w1s, w2, w2s, b1, b2, hp, ip = cases.padded_device_weights(L)
+    assert (hp, ip) == (160, 224)
+    tw, ti = torch.from_numpy(L.topk_w).cuda(), torch.from_numpy(L.topk_ids).cuda()
+    print(f"unfetched-padding case T={T} bm={bm}", flush=True)
+    kw = dict(w1_scale=w1s, w2_scale=w2s, block_size_M=bm, bias1=b1, bias2=b2, dtype=torch.float32, method="a4w4")
+    wide = torch.nn.functional.pad(L.hidden, (0, hp)).cuda()
+    told = fused_moe(wide, w1, w2, tw, ti, hidden_pad=hp, intermediate_pad=ip, **kw)
+    told_steps, parts = fused_moe(wide, w1, w2, tw, ti, hidden_pad=hp, intermediate_pad=ip, return_parts=True, **kw)
+    untold = fused_moe(wide, w1, w2, tw, ti, **kw)
+    torch.cuda.synchronize()
+    assert told.shape == (T, L.H + hp) and torch.equal(told, untold) and torch.equal(told_steps, untold)
+    assert (_f(told)[:, L.H:] == 0).all()
+    nv = int(parts["num_valid_ids"][0])
+    assert (_f(parts["a2"])[:nv, L.I:] == 0).all() and (_f(parts["out3"])[:, :, L.H:] == 0).all()
+    ref = moe.moe_ref(_f(L.hidden), L.w1q, L.w1s, L.w2q, L.w2s, L.topk_w, L.topk_ids, act="a4", bias1=_f(L.bias1),
+                      bias2=_f(L.bias2))
+    view = dict(parts, a2=parts["a2"][:, :L.I], out3=parts["out3"][:, :, :L.H])
+    w1e, w2e, ref_a2, nflip1 = _stage_checks(L, view, parts["block_m"])
+    assert w1e <= TOL_MAX and w2e <= TOL_MAX
+    _end_to_end(_f(told)[:, :L.H], ref, ref_a2, nflip1)
+
+
 @pytest.mark.parametrize("name,T,bm,bias,splitk", [
     ("tiny", 64, 16, False, 1), ("tiny", 5, 16, True, 0), ("tiny", 200, 64, False, 1), ("mixtral_s", 33, 32, False, 1),
     ("qwen3_s", 64, 16, False, 1), ("dsv3_s", 16, None, False, 1), ("dsv3_s", 128, None, True, 1),

@@ -27,7 +27,7 @@ def _both(lib, L, dev_w, w4a16, bm, nl=None):
     stream = _lib.current_stream()
     common = (_lib.dptr(hidden), H, _lib.dptr(w1), _lib.dptr(w1s), _lib.dptr(w2), _lib.dptr(w2s), None, None,
               _lib.dptr(ti), _lib.dptr(tw), None, _lib.dptr(nl))
-    tail = (0, T, k, E, H, I, bm, w4a16, 0, 0, 0.0)
+    tail = (0, T, k, E, H, I, 0, 0, bm, w4a16, 0, 0, 0.0)
     out_a = torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
     out_b = torch.full((T, H), float("nan"), dtype=torch.bfloat16, device="cuda")
     ws_bytes = lib.pyhip_moe_forward_workspace_bytes(T, k, E, H, I, bm, w4a16)
@@ -61,7 +61,7 @@ def test_static_scratch_entry_point_rejects_oversized_calls():
     assert cap() == 64 << 20
     one = ctypes.c_void_p(256)
     # DeepSeek-V3 shape, 8192 tokens: far more intermediates than the array holds; refused before anything is launched
-    rc = fn(one, 7168, one, one, one, one, None, None, one, one, None, None, one, 0, 8192, 8, 256, 7168, 2048, 128, 0, 0, 0,
+    rc = fn(one, 7168, one, one, one, one, None, None, one, one, None, None, one, 0, 8192, 8, 256, 7168, 2048, 0, 0, 128, 0, 0, 0,
             0.0, None)
     assert rc == 1 and b"scratch array holds" in lib.pyhip_moe_last_error()
 
@@ -76,7 +76,7 @@ def _prepared_call(lib, L, dev_w, w4a16, bm):
     out = torch.full((L.T, L.H), float("nan"), dtype=torch.bfloat16, device="cuda")
     keep = (hidden, tw, ti, w1, w1s, w2, w2s)
     args = (_lib.dptr(hidden), L.H, _lib.dptr(w1), _lib.dptr(w1s), _lib.dptr(w2), _lib.dptr(w2s), None, None,
-            _lib.dptr(ti), _lib.dptr(tw), None, None, _lib.dptr(out), 0, L.T, L.k, L.E, L.H, L.I, bm, w4a16, 0, 0, 0.0)
+            _lib.dptr(ti), _lib.dptr(tw), None, None, _lib.dptr(out), 0, L.T, L.k, L.E, L.H, L.I, 0, 0, bm, w4a16, 0, 0, 0.0)
 
     def call():
         _lib.check(fn(*args, _lib.current_stream()), "moe_forward_static")
