@@ -234,6 +234,25 @@ int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t*
                           const uint32_t* num_valid_ids, void* out3_bf16, int tokens, int topk, int experts,
                           int hidden, int inter, int block_m, int64_t n_blk, int split_k, pyhip_stream_t stream);
 
+/* The same two GEMMs for a single token, without the routing sort in front of them: the kernels read the token's
+ * topk_ids [topk] / topk_weights [topk] themselves, one 16-row block per slot, and apply the sort's drop rule
+ * (expert id outside [0, experts), masked expert, *num_local_tokens < 1) and the local expert numbering under an
+ * expert mask.  The reference's decode path runs its sort for every token count (src/contrib/fused_moe.py:283-305);
+ * at one token the sort is a launch of 6 us on the critical path of a layer of 40-50 us.
+ *   a2    bf16 [topk * 16, inter]: slot s is row 16 * s (what a sort with block_size 16 gives when every slot has an
+ *         expert of its own)
+ *   out3  bf16 [1, topk, hidden]; dropped slots are left unwritten, as by pyhip_moe_gemm2_w4a16
+ * Results equal those of pyhip_moe_sorting + pyhip_moe_gemm{1,2}_w4a16 bit for bit.  pyhip_moe_forward takes this
+ * path by itself for tokens == 1 with bf16 activations. */
+int pyhip_moe_gemm1_w4a16_token(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale,
+                                const void* bias1_bf16, const int32_t* topk_ids, const int32_t* expert_mask,
+                                const int32_t* num_local_tokens, void* a2_bf16, int topk, int experts, int hidden,
+                                int inter, int split_k, int activation, float swiglu_limit, pyhip_stream_t stream);
+int pyhip_moe_gemm2_w4a16_token(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale, const void* bias2_bf16,
+                                const int32_t* topk_ids, const float* topk_weights, const int32_t* expert_mask,
+                                const int32_t* num_local_tokens, void* out3_bf16, int topk, int experts, int hidden,
+                                int inter, int split_k, pyhip_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Top-k reduction out[t, :] = sum_slot in[t, slot, :] (fp32, slots in index order), one rounding.
  * Replaces moe_gemm_final_reduce_bf16, src/contrib/moe_gemm_mxfp4.py:199-282

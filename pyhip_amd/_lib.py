@@ -46,6 +46,8 @@ SIGNATURES = {
                                           _I, _I, _I, _I, _I, _I, _L, _P]),
     "pyhip_moe_gemm1_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _P]),
     "pyhip_moe_gemm2_w4a16": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _P]),
+    "pyhip_moe_gemm1_w4a16_token": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P]),
+    "pyhip_moe_gemm2_w4a16_token": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "pyhip_moe_probe_mfma_stream": (_I, [_I, _I, _P, _L, _P, _I, _P, _P]),
     "pyhip_moe_topk_reduce": (_I, [_P, _P, _L, _I, _I, _I, _P, _P]),
     "pyhip_moe_topk_reduce_routed": (_I, [_P, _P, _L, _I, _I, _I, _P, _I, _P, _P, _P]),

@@ -15,4 +15,4 @@ extern "C" void pyhip_set_error(const char* fmt, ...)
 
 extern "C" const char* pyhip_moe_last_error(void) { return g_last_error; }
 
-extern "C" int pyhip_moe_abi_version(void) { return 8; }
+extern "C" int pyhip_moe_abi_version(void) { return 9; }

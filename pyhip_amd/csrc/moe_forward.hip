@@ -24,6 +24,10 @@ int pyhip_moe_gemm1_w4a16(const void*, const uint8_t*, const uint8_t*, const voi
                           const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, int, float, hipStream_t);
 int pyhip_moe_gemm2_w4a16(const void*, const uint8_t*, const uint8_t*, const void*, const uint32_t*, const float*,
                           const uint32_t*, const uint32_t*, void*, int, int, int, int, int, int, int64_t, int, hipStream_t);
+int pyhip_moe_gemm1_w4a16_token(const void*, const uint8_t*, const uint8_t*, const void*, const int32_t*, const int32_t*,
+                                const int32_t*, void*, int, int, int, int, int, int, float, hipStream_t);
+int pyhip_moe_gemm2_w4a16_token(const void*, const uint8_t*, const uint8_t*, const void*, const int32_t*, const float*,
+                                const int32_t*, const int32_t*, void*, int, int, int, int, int, hipStream_t);
 int pyhip_moe_route_sorting(const float*, int, int, int, int, int, int, int, const int32_t*, const int32_t*, float*, int32_t*,
                             uint32_t*, float*, uint32_t*, uint32_t*, uint32_t*, void*, int64_t, const void*, int64_t, int64_t,
                             int, uint8_t*, uint8_t*, hipStream_t);
@@ -200,6 +204,20 @@ static int forward_impl(const void* hidden_bf16, int64_t hidden_row_stride, cons
     uint32_t* sched   = (uint32_t*)(ws + l.sched);
     void* out3        = ws + l.out3;
     int rc;
+    if(w4a16 && tokens == 1 && !router.gating)
+    {
+        // a single token with bf16 activations: no sort; the GEMMs read the routing themselves, one block per slot
+        rc = pyhip_moe_gemm1_w4a16_token(hidden_bf16, w1, w1_scale, bias1_bf16, topk_ids, expert_mask, num_local_tokens,
+                                         ws + l.a2, topk, experts, hidden, inter, split_k, activation, swiglu_limit, stream);
+        if(rc)
+            return rc;
+        rc = pyhip_moe_gemm2_w4a16_token(ws + l.a2, w2, w2_scale, bias2_bf16, topk_ids, topk_weights, expert_mask,
+                                         num_local_tokens, out3, topk, experts, hidden, inter, split_k, stream);
+        if(rc)
+            return rc;
+        return pyhip_moe_topk_reduce_routed(out3, out, tokens, topk, hidden, out_is_f32, topk_ids, experts, expert_mask,
+                                            num_local_tokens, stream);
+    }
     if(router.gating)
         // the routing is part of the call: the sort's own workgroup routes the tokens when there are few of them
         rc = pyhip_moe_route_sorting(router.gating, tokens, topk, experts, router.n_group, router.topk_group,

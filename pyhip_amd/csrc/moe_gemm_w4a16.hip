@@ -36,6 +36,14 @@ struct W4A16Args
     uint16_t* out;             // stage 1: bf16 [n_blk*BM, N/2]; stage 2: bf16 [T, topk, N]
     int T, topk, K, N, SC, n_tiles;
     GatedAct act;              // stage 1: the gated activation (common.h)
+    // One token, no sort (the *_token entry points): block b is the token's slot b, with one real row.  The kernels read
+    // the routing themselves: the expert of the slot, whether the slot takes part (the sort's drop rule) and the local
+    // id of its expert under an expert mask.  sorted_ids / sorted_w / sorted_e / num_valid are not used then.
+    const int* token_ids     = nullptr;   // [topk] expert ids of the token's slots
+    const float* token_w     = nullptr;   // [topk] routing weights (stage 2)
+    const int* expert_mask   = nullptr;   // [experts] or null
+    const int* num_local_tok = nullptr;   // device scalar or null: 0 = the token is not this rank's
+    int experts              = 0;
 };
 
 // 32 e2m1 values (4 dwords) times 2^(scale byte - 127) -> four MFMA operands of 8 bf16
@@ -65,9 +73,36 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int r = lane & 15, kb = lane >> 4;
     const int m_blk = blockIdx.x / g.n_tiles, nt = blockIdx.x - m_blk * g.n_tiles;
-    if((u32)(m_blk * BM) >= g.num_valid[0])
-        return;
-    const int e  = (int)g.sorted_e[m_blk];
+    const bool one_token = g.token_ids != nullptr;
+    int e;
+    if(one_token)
+    {
+        if(m_blk >= g.topk || (g.num_local_tok && *g.num_local_tok < 1))
+            return;
+        const int eg = g.token_ids[m_blk];
+        if(!moe_pair_is_kept(eg, g.experts, g.expert_mask))
+            return;
+        e = eg;
+        if(g.expert_mask)                     // local id: the experts this rank holds before this one
+        {
+            e = 0;
+            for(int i0 = 0; i0 < eg; i0 += WAVE)
+                e += __builtin_popcountll(__ballot(i0 + lane < eg && g.expert_mask[i0 + lane] != 0));
+            e = __builtin_amdgcn_readfirstlane(e);
+        }
+    }
+    else
+    {
+        if((u32)(m_blk * BM) >= g.num_valid[0])
+            return;
+        e = (int)g.sorted_e[m_blk];
+    }
+    // sorted id of position p: (slot << 24) | token; positions without a row carry slot = topk
+    auto sorted_id = [&](int p) __attribute__((always_inline)) -> u32 {
+        if(one_token)
+            return p == m_blk * BM ? (u32)m_blk << 24 : ((u32)g.topk << 24) | (u32)g.T;
+        return g.sorted_ids[p];
+    };
     const int Kb = g.K / 2, I = g.N / 2;
     // first output channel of this wave's rows (stage 1: within the gate half; the up half is I further)
     const int chbase = STAGE == 1 ? (SPLITK ? nt * 32 : nt * 128 + wave * 32) : (SPLITK ? nt * 64 : nt * 256 + wave * 64);
@@ -90,12 +125,12 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     const uint16_t* ap[MT];
     bool ok[MT];
     u32 ids[MT];
-    const int tok0 = STAGE == 1 ? (int)(g.sorted_ids[m_blk * BM] & 0xFFFFFFu) : 0;
+    const int tok0 = STAGE == 1 ? (int)(sorted_id(m_blk * BM) & 0xFFFFFFu) : 0;
 #pragma unroll
     for(int mt = 0; mt < MT; mt++)
     {
         const int p  = m_blk * BM + mt * 16 + r;
-        ids[mt]      = g.sorted_ids[p];
+        ids[mt]      = sorted_id(p);
         const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
         ok[mt]       = slot < g.topk && tok < g.T;
         // padding rows compute nothing that is stored: they all read the row of the block's first position, which
@@ -226,7 +261,7 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
         else if(ok[mt])
         {
             const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
-            const float rw = g.sorted_w[p];
+            const float rw = one_token ? g.token_w[m_blk] : g.sorted_w[p];
 #pragma unroll
             for(int j = 0; j < 4; j++)
             {
@@ -319,6 +354,62 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
     g.SC = (hidden / 32 + 7) / 8 * 8; g.n_tiles = inter / 128;
     g.act = make_gated_act(activation, swiglu_limit);
     return launch_w4a16<1>(g, block_m, n_blk, (int64_t)tokens * topk, experts, split_k, stream);
+}
+
+// The two GEMMs for a single token without the routing sort: the kernels read topk_ids / topk_weights themselves, one
+// 16-row block per slot (the rows of a2 and the blocks are those a sort with block_size 16 would produce when every
+// slot has an expert of its own: a2 bf16 [topk * 16, inter], row slot * 16).  Slots the sort would drop (expert id outside
+// [0, experts), masked expert, num_local_tokens < 1) are left out; their out3 rows keep what the buffer held, as
+// with the sorted entry points.  One launch fewer on the critical path of single-token decode, where the sort's 6 us
+// are an eighth of the layer.  Results are those of the sorted entry points, bit for bit.
+extern "C" int pyhip_moe_gemm1_w4a16_token(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale,
+                                           const void* bias1_bf16, const int32_t* topk_ids, const int32_t* expert_mask,
+                                           const int32_t* num_local_tokens, void* a2_bf16, int topk, int experts,
+                                           int hidden, int inter, int split_k, int activation, float swiglu_limit,
+                                           hipStream_t stream)
+{
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm1_w4a16_token: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
+                  "moe_gemm1_w4a16_token: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
+    PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && topk_ids && a2_bf16, "moe_gemm1_w4a16_token: null pointer");
+    PYHIP_REQUIRE(hidden > 0 && hidden % 512 == 0 && inter > 0 && inter % 128 == 0,
+                  "moe_gemm1_w4a16_token: hidden=%d must be a multiple of 512, inter=%d of 128", hidden, inter);
+    PYHIP_REQUIRE(topk > 0 && topk < 256 && experts > 0, "moe_gemm1_w4a16_token: bad sizes");
+    PYHIP_REQUIRE(((uintptr_t)hidden_bf16 % 16) == 0 && ((uintptr_t)w1 % 16) == 0 && ((uintptr_t)w1_scale % 4) == 0 &&
+                      ((uintptr_t)a2_bf16 % 8) == 0,
+                  "moe_gemm1_w4a16_token: unaligned pointer");
+    W4A16Args g;
+    g.a = (const uint16_t*)hidden_bf16; g.w = w1; g.w_s = w1_scale; g.bias = (const uint16_t*)bias1_bf16;
+    g.sorted_ids = nullptr; g.sorted_w = nullptr; g.sorted_e = nullptr; g.num_valid = nullptr;
+    g.out = (uint16_t*)a2_bf16; g.T = 1; g.topk = topk; g.K = hidden; g.N = 2 * inter;
+    g.SC = (hidden / 32 + 7) / 8 * 8; g.n_tiles = inter / 128;
+    g.act = make_gated_act(activation, swiglu_limit);
+    g.token_ids = topk_ids; g.expert_mask = expert_mask; g.num_local_tok = num_local_tokens; g.experts = experts;
+    return launch_w4a16<1>(g, 16, topk, topk, experts, split_k, stream);
+}
+
+extern "C" int pyhip_moe_gemm2_w4a16_token(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale,
+                                           const void* bias2_bf16, const int32_t* topk_ids, const float* topk_weights,
+                                           const int32_t* expert_mask, const int32_t* num_local_tokens, void* out3_bf16,
+                                           int topk, int experts, int hidden, int inter, int split_k, hipStream_t stream)
+{
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm2_w4a16_token: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(a2_bf16 && w2 && w2_scale && topk_ids && topk_weights && out3_bf16, "moe_gemm2_w4a16_token: null pointer");
+    PYHIP_REQUIRE(inter > 0 && inter % 512 == 0 && hidden > 0 && hidden % 256 == 0,
+                  "moe_gemm2_w4a16_token: inter=%d must be a multiple of 512, hidden=%d of 256", inter, hidden);
+    PYHIP_REQUIRE(topk > 0 && topk < 256 && experts > 0, "moe_gemm2_w4a16_token: bad sizes");
+    PYHIP_REQUIRE(((uintptr_t)a2_bf16 % 16) == 0 && ((uintptr_t)w2 % 16) == 0 && ((uintptr_t)w2_scale % 4) == 0 &&
+                      ((uintptr_t)out3_bf16 % 8) == 0,
+                  "moe_gemm2_w4a16_token: unaligned pointer");
+    W4A16Args g;
+    g.a = (const uint16_t*)a2_bf16; g.w = w2; g.w_s = w2_scale; g.bias = (const uint16_t*)bias2_bf16;
+    g.sorted_ids = nullptr; g.sorted_w = nullptr; g.sorted_e = nullptr; g.num_valid = nullptr;
+    g.out = (uint16_t*)out3_bf16; g.T = 1; g.topk = topk; g.K = inter;
+    g.N = hidden; g.SC = (inter / 32 + 7) / 8 * 8; g.n_tiles = hidden / 256;
+    g.act = make_gated_act(0, 0.f);
+    g.token_ids = topk_ids; g.token_w = topk_weights; g.expert_mask = expert_mask; g.num_local_tok = num_local_tokens;
+    g.experts = experts;
+    return launch_w4a16<2>(g, 16, topk, topk, experts, split_k, stream);
 }
 
 extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, const uint8_t* w2_scale,

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_lib.SIGNATURES) == names
-    assert lib.pyhip_moe_abi_version() == 8
+    assert lib.pyhip_moe_abi_version() == 9
 
 
 def test_size_helpers():

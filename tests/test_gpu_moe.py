@@ -487,6 +487,61 @@ def test_expert_mask_and_local_tokens(method, T):
     assert (out[n_local:] == 0).all()
 
 
+@pytest.mark.parametrize("name,bias,swiglu", [("mixtral_s", False, False), ("dsv3_s", True, False), ("tiny", True, True),
+                                              ("longk_s", False, False)])
+def test_single_token_skips_the_sort(name, bias, swiglu):
+    """One token with bf16 activations: the layer call runs no sort, the GEMMs read topk_ids / topk_weights themselves
+    (pyhip_moe_gemm{1,2}_w4a16_token).  The result must equal the sorted, step-by-step path bit for bit (which the
+    other tests hold against the oracle): plain, with an out-of-range id, under an expert mask with the rank's own
+    weights only (local expert numbering), and with num_local_tokens 0 and 1; also on poisoned intermediates."""
+    from pyhip_amd.enums import ActivationType
+    L = cases.make_layer(name, 1, seed=41, bias=bias)
+    w1, w1s, w2, w2s = cases.device_weights(L)
+    hidden = L.hidden.cuda()
+    tw = torch.from_numpy(L.topk_w).cuda()
+    b1 = None if L.bias1 is None else L.bias1.cuda()
+    b2 = None if L.bias2 is None else L.bias2.cuda()
+    act = dict(activation=ActivationType.Swiglu, swiglu_limit=7.0) if swiglu else {}
+    E = L.E
+    s1, s2 = w1s.view(E, -1), w2s.view(E, -1)
+    print(f"single-token case {name} bias={bias} swiglu={swiglu}", flush=True)
+    ids_plain = L.topk_ids.copy()
+    ids_hole = ids_plain.copy()
+    ids_hole[0, 0] = E + 3                                      # a slot whose expert lives elsewhere
+    ran = 0
+    for ids in (ids_plain, ids_hole):
+        ti = torch.from_numpy(ids).cuda()
+        for masked in (False, True):
+            kw = dict(w1_scale=w1s, w2_scale=w2s, bias1=b1, bias2=b2, method="w4a16", **act)
+            wa, wb = w1, w2
+            if masked:
+                # the rank holds every expert but the one of the token's last slot, and none beyond the 3/4 mark
+                mask = torch.ones(E, dtype=torch.int32)
+                mask[int(L.topk_ids[0, -1])] = 0
+                mask[(3 * E) // 4:] = 0
+                if int(mask[torch.from_numpy(ids_plain[0]).long().clamp(0, E - 1)].sum()) == 0:
+                    mask[int(L.topk_ids[0, 0])] = 1
+                keep = mask.bool().cuda()
+                wa, wb = w1[keep].contiguous(), w2[keep].contiguous()
+                wa.is_shuffled = wb.is_shuffled = True
+                kw.update(expert_mask=mask.cuda(), w1_scale=s1[keep].contiguous().view(-1, w1s.shape[-1]),
+                          w2_scale=s2[keep].contiguous().view(-1, w2s.shape[-1]),
+                          bias1=None if b1 is None else b1[keep].contiguous(), bias2=None if b2 is None else b2[keep].contiguous())
+            for nl in (None, 1, 0):
+                if nl is not None:
+                    kw["num_local_tokens"] = torch.tensor([nl], dtype=torch.int32, device="cuda")
+                for dt in (torch.float32, torch.bfloat16):
+                    want = fused_moe(hidden, wa, wb, tw, ti, dtype=dt, return_parts=True, **kw)[0]
+                    _poison_allocator(8 << 20)
+                    got = fused_moe(hidden, wa, wb, tw, ti, dtype=dt, **kw)
+                    torch.cuda.synchronize()
+                    assert torch.isfinite(got.float()).all() and torch.equal(got, want), (masked, nl, dt)
+                    if nl == 0:
+                        assert (got == 0).all()
+                    ran += 1
+    assert ran == 24
+
+
 @pytest.mark.parametrize("method", ["a4w4", "w4a16"])
 def test_strided_hidden_states(method):
     """hidden_states may be a column slice of a wider tensor (row stride larger than the hidden size): the result
