@@ -212,6 +212,24 @@ def test_last_arriver_reduce_at_full_size(layer, T, bm):
         assert torch.equal(got, want), rep
 
 
+@pytest.mark.parametrize("layer", ["mixtral", "gptoss", "dsv3"], indirect=True)
+def test_single_token_without_the_sort_at_full_size(layer):
+    """One token at the benchmark shapes: the layer call takes the bf16-activation kernels and skips the sort (the GEMMs
+    read the routing themselves); the result must equal the sorted, step-by-step path bit for bit, and method "auto"
+    must be that same path."""
+    W = layer
+    from pyhip_amd import workloads
+    hidden, tw, ti = workloads.make_inputs(W["shape"], 1)
+    print(f"full-size single-token case {W['shape']}", flush=True)
+    for dt in (torch.bfloat16, torch.float32):
+        want = _run(W, hidden, tw, ti, method="w4a16", dtype=dt, return_parts=True)[0]
+        got = _run(W, hidden, tw, ti, method="w4a16", dtype=dt)
+        auto = _run(W, hidden, tw, ti, method="auto", dtype=dt)
+        torch.cuda.synchronize()
+        assert torch.isfinite(got.float()).all() and got.float().abs().max() > 0
+        assert torch.equal(got, want) and torch.equal(auto, got)
+
+
 @pytest.mark.parametrize("layer", ["dsv3"], indirect=True)
 @pytest.mark.parametrize("T,bms", [(1024, (16, 32, 64, 128, 256)), (4096, (64, 128, 160, 192, 256)), (5120, (128, 192, 288))])
 def test_load_policies_agree_bit_for_bit(layer, T, bms):
