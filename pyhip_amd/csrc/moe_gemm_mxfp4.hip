@@ -22,8 +22,8 @@
 #include "gemm_device.h"
 
 // most experts a persistent launch can serve: the schedule (E + 1 block prefixes, E local ids) sits in LDS next to the
-// activation stages, and two workgroups of the 128-row tile must still fit one CU (2 x 80 KB), four of the 16-row
-// tile (4 x 40 KB)
+// activation stages, and two workgroups of the 128-row tile must still fit one CU (2 x 80 KB), three of the 16-row
+// tile (40 KB each)
 #define SCHED_E_MAX 704
 #define SCHED_E_MAX_16 512
 
@@ -620,11 +620,13 @@ static int launch_gemm(GemmArgs g, int block_m, int act, hipStream_t stream, boo
         g.sched = nullptr;
     if(g.sched)
     {
-        // persistent: as many workgroups per CU as fit (four of the 16-row tile: 4 x 40 KB of LDS, 128 registers; three of
-        // the 32-row tile; two up to 128 rows; one of the 256-row tile).  The small tiles are bound by the weight stream;
-        // what the further workgroups buy is more loads in flight and fewer, fuller rounds when the tiles number little more
-        // than the resident workgroups (DeepSeek-V3 shape at 16 tokens: 0.417 ms with two, 0.378 with three, 0.377 with
-        // four; gpt-oss shape at 16 tokens 0.139 -> 0.133 ms with the fourth)
+        // persistent: as many workgroups per CU as fit (three of the 16- and 32-row tiles: 136-160 registers, 40 KB of LDS;
+        // two up to 128 rows; one of the 256-row tile).  The small tiles are bound by the weight stream; what the further
+        // workgroups buy is more loads in flight (DeepSeek-V3 shape at 16 tokens: 0.417 ms with two per CU, 0.378 with
+        // three).  The 16-row tile is launched with four per CU although only three are resident at a time: the last
+        // quarter of the grid starts as the first workgroups leave (per-workgroup time stamps show it) and fills the
+        // slots they free with its own, smaller shares of the tile list, which evens out the end of the launch
+        // (DeepSeek-V3 shape at 16 tokens 0.378 -> 0.377 ms, gpt-oss shape at 16 tokens 0.139 -> 0.133 ms)
         const int cus = device_cu_count();
         unsigned resident = (unsigned)cus * (block_m == 16 ? 4u : block_m <= 32 ? 3u : block_m <= 128 ? 2u : 1u) / 8u * 8u;
         nwg               = nwg < resident ? (nwg + 7u) / 8u * 8u : resident;
