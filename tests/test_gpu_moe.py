@@ -269,6 +269,60 @@ def test_padding_is_left_unfetched_and_changes_nothing(T, bm):
     _end_to_end(_f(told)[:, :L.H], ref, ref_a2, nflip1)
 
 
+@pytest.mark.parametrize("T,bm", [(24, 16), (300, 128), (500, 288)])
+def test_padded_weight_rows_are_not_read(T, bm):
+    """Whether the kernels really leave the padding alone: hidden 1408 (22 x 64) and inter 1312 (41 x 32) padded to
+    1536, and the weight rows of the padding (whole waves' worth in both GEMMs) filled with ones instead of zeros,
+    which a caller must not do.  Told the pads, the GEMMs do not fetch those rows: the padded columns of a2, out3 and
+    the output are exact zeros and everything equals the run on clean weights.  Not told, the ones show up."""
+    from oracle import layout
+    from pyhip_amd import mxfp4 as pm
+    L = cases.make_layer("gptoss_s", T, seed=6, H=1408, I=1312)
+    t = torch.from_numpy
+    w1q, w1s, w2q, w2s, _, _, hp, ip = pm.pad_layer_weights(t(L.w1q), t(L.w1s), t(L.w2q), t(L.w2s))
+    assert (hp, ip) == (128, 224)
+    E, H, I, Hp, Ip = L.E, L.H, L.I, L.H + hp, L.I + ip
+
+    def device(w1q, w1s, w2q, w2s):
+        w1 = t(layout.shuffle_weight(w1q.numpy())).cuda()
+        w2 = t(layout.shuffle_weight(w2q.numpy())).cuda()
+        s1 = t(layout.e8m0_shuffle(w1s.numpy().reshape(E * 2 * Ip, Hp // 32))).cuda()
+        s2 = t(layout.e8m0_shuffle(w2s.numpy().reshape(E * Hp, Ip // 32))).cuda()
+        w1.is_shuffled = w2.is_shuffled = True
+        return w1, s1, w2, s2
+
+    clean = device(w1q, w1s, w2q, w2s)
+    d1q, d1s, d2q, d2s = w1q.clone(), w1s.clone(), w2q.clone(), w2s.clone()
+    for lo, hi in ((I, Ip), (Ip + I, 2 * Ip)):            # the padding rows of the gate half and of the up half
+        d1q[:, lo:hi, : H // 2] = 0x22                      # e2m1 pairs (1.0, 1.0), over the real columns
+        d1s[:, lo:hi, : H // 32] = 127                      # scale 2^0
+    d2q[:, H:, : I // 2] = 0x22
+    d2s[:, H:, : I // 32] = 127
+    dirty = device(d1q, d1s, d2q, d2s)
+    tw, ti = t(L.topk_w).cuda(), t(L.topk_ids).cuda()
+    wide = torch.nn.functional.pad(L.hidden, (0, hp)).cuda()
+    print(f"unread-padding case T={T} bm={bm}", flush=True)
+
+    def run(w, **pads):
+        w1, s1, w2, s2 = w
+        return fused_moe(wide, w1, w2, tw, ti, w1_scale=s1, w2_scale=s2, block_size_M=bm, dtype=torch.float32, method="a4w4",
+                         return_parts=True, **pads)
+
+    want, pw = run(clean, hidden_pad=hp, intermediate_pad=ip)
+    got, pg = run(dirty, hidden_pad=hp, intermediate_pad=ip)
+    seen, ps = run(dirty)
+    one_call = fused_moe(wide, dirty[0], dirty[2], tw, ti, w1_scale=dirty[1], w2_scale=dirty[3], block_size_M=bm,
+                         dtype=torch.float32, method="a4w4", hidden_pad=hp, intermediate_pad=ip)
+    torch.cuda.synchronize()
+    nv = int(pg["num_valid_ids"][0])
+    assert torch.equal(got, want) and torch.equal(one_call, want)
+    assert (got[:, H:] == 0).all() and (_f(pg["a2"])[:nv, I:] == 0).all() and (_f(pg["out3"])[:, :, H:] == 0).all()
+    assert torch.equal(pg["a2"][:nv], pw["a2"][:nv]) and torch.equal(pg["out3"], pw["out3"])
+    # the poison is there to be seen by kernels that fetch everything
+    assert (_f(ps["a2"])[:nv, I:] != 0).any() and (seen[:, H:] != 0).any()
+    assert torch.equal(seen[:, :H], want[:, :H])
+
+
 @pytest.mark.parametrize("name,T,bm,bias,splitk", [
     ("tiny", 64, 16, False, 1), ("tiny", 5, 16, True, 0), ("tiny", 200, 64, False, 1), ("mixtral_s", 33, 32, False, 1),
     ("qwen3_s", 64, 16, False, 1), ("dsv3_s", 16, None, False, 1), ("dsv3_s", 128, None, True, 1),
