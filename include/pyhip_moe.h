@@ -222,8 +222,9 @@ int pyhip_moe_gemm2_mxfp4_reduce(const uint8_t* a2_q, const uint8_t* a2_scale, c
  * adding into the layer output with atomics.  block_m is 16, 32 or 64; hidden % 512 == 0, inter % 512 == 0.
  * split_k: 4 = the four waves of a workgroup share a 64-row weight tile and split K between them (partial sums
  * meet in LDS; four times as many workgroups), 16 = the same with sixteen waves per workgroup (block_m = 16,
- * K >= 2048), 1 = every wave owns 64 rows over the whole K, 0 = split when the launch would otherwise have fewer
- * than 2048 workgroups with work, sixteen-fold when even then fewer workgroups than CUs would start and K >= 8192.  activation / swiglu_limit: as for
+ * K >= 2048), 32 = sixteen waves share a 32-row weight tile and keep three K-steps in flight (down GEMM; block_m = 16,
+ * K >= 2048; the gate_up GEMM takes 16 instead), 1 = every wave owns 64 rows over the whole K, 0 = split when the launch would otherwise have fewer
+ * than 2048 workgroups with work, sixteen-fold (the down GEMM: split 32) when even then fewer workgroups than CUs would start and K >= 8192.  activation / swiglu_limit: as for
  * pyhip_moe_gemm1_mxfp4. */
 int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1, const uint8_t* w1_scale, const void* bias1_bf16,
                           const uint32_t* sorted_ids, const uint32_t* sorted_expert_ids, const uint32_t* num_valid_ids,

@@ -63,12 +63,23 @@ __device__ __forceinline__ void expand_fp4(const v4i& w, u32 scale_byte, v8bf (&
 }
 
 // STAGE 1 = gate_up (+ SiLU(gate) * up), 2 = down (* routing weight).  MT = row groups of 16 per tile.
+// SPLIT = 0: every wave owns 64 weight rows over the whole K.  4 / 16: that many waves share a 64-row weight tile and
+// split K.  32 (down GEMM only): sixteen waves share a 32-row weight tile, and every wave keeps three K-steps of
+// operands in flight instead of two.  For the down GEMM of a layer with few experts and a long K at one or two tokens
+// (Mixtral shape: 2 experts x 16 tiles of 256 rows, K = 14336) the sixteen-wave split starts 128 workgroups on 256 CUs,
+// and a wave walks its seven K-steps one memory latency at a time; half as wide a tile fills the chip, and the
+// narrower tile leaves the registers for the third K-step.
 template <int STAGE, int MT, int SPLIT>
-__global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
+__global__ void __launch_bounds__(SPLIT >= 16 ? 1024 : W4A16_THREADS) moe_gemm_w4a16_kernel(W4A16Args g)
 {
     constexpr int BM      = MT * 16;
     constexpr bool SPLITK = SPLIT != 0;
-    __shared__ float red[SPLITK ? SPLIT * 4 * MT * WAVE * 4 : 1];  // [wave][j][mt][lane][4]
+    constexpr bool DEEP   = SPLIT == 32;
+    constexpr int NW      = DEEP ? 16 : SPLIT;    // waves that split K
+    constexpr int RG      = DEEP ? 2 : 4;         // 16-row weight row groups of a wave
+    constexpr int NB      = DEEP ? 3 : 2;         // K-steps of operands in registers
+    static_assert(!DEEP || STAGE == 2, "the 32-row tile exists for the down GEMM");
+    __shared__ float red[SPLITK ? NW * RG * MT * WAVE * 4 : 1];  // [wave][j][mt][lane][4]
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int r = lane & 15, kb = lane >> 4;
@@ -105,15 +116,15 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     };
     const int Kb = g.K / 2, I = g.N / 2;
     // first output channel of this wave's rows (stage 1: within the gate half; the up half is I further)
-    const int chbase = STAGE == 1 ? (SPLITK ? nt * 32 : nt * 128 + wave * 32) : (SPLITK ? nt * 64 : nt * 256 + wave * 64);
+    const int chbase = STAGE == 1 ? (SPLITK ? nt * 32 : nt * 128 + wave * 32) : (SPLITK ? nt * (16 * RG) : nt * 256 + wave * 64);
 
     // weight row groups of this wave: j = 0..3 (stage 1: j>>1 selects gate / up)
-    const uint8_t* wp[4];
-    const uint8_t* sp[4];      // scale tile row (32 weight rows) of row group j
-    int sbyte_row[4];          // which 16-row half of the 32-row scale tile
+    const uint8_t* wp[RG];
+    const uint8_t* sp[RG];     // scale tile row (32 weight rows) of row group j
+    int sbyte_row[RG];         // which 16-row half of the 32-row scale tile
     const size_t sc_tile = (size_t)(g.SC / 8) * 256;
 #pragma unroll
-    for(int j = 0; j < 4; j++)
+    for(int j = 0; j < RG; j++)
     {
         const size_t row = STAGE == 1 ? (size_t)e * g.N + (j >> 1) * I + chbase + (j & 1) * 16
                                       : (size_t)e * g.N + chbase + j * 16;
@@ -140,26 +151,26 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
         ap[mt]       = g.a + row * g.K + kb * 32;
     }
 
-    v4f acc[4][MT];
+    v4f acc[RG][MT];
 #pragma unroll
-    for(int j = 0; j < 4; j++)
+    for(int j = 0; j < RG; j++)
 #pragma unroll
         for(int mt = 0; mt < MT; mt++)
             acc[j][mt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     const int KT = g.K / 128;
-    constexpr int KSTRIDE = SPLITK ? SPLIT : 1;
-    v4i wf[2][4];
-    v4i af[2][MT][4];
-    u32 wsc[2][4];             // scale dwords (one covers the two K-steps of a 256-K column tile), loaded with
+    constexpr int KSTRIDE = SPLITK ? NW : 1;
+    v4i wf[NB][RG];
+    v4i af[NB][MT][4];
+    u32 wsc[NB][RG];           // scale dwords (one covers the two K-steps of a 256-K column tile), loaded with
                                // the K-step's weights: fetched only when needed, their latency would add to every step
     auto load_step = [&](auto BB, int kt) __attribute__((always_inline)) {
         constexpr int buf = decltype(BB)::value;
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
             wsc[buf][j] = *(const u32*)(sp[j] + (size_t)(kt >> 1) * 256);
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
             wf[buf][j] = __builtin_nontemporal_load((const v4i*)(wp[j] + (size_t)kt * 1024));
 #pragma unroll
         for(int mt = 0; mt < MT; mt++)
@@ -167,13 +178,11 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
             for(int i = 0; i < 4; i++)
                 af[buf][mt][i] = *(const v4i*)(ap[mt] + kt * 128 + i * 8);
     };
-    // one K-step from register set P while the next one loads into set 1 - P (K / 128 is even)
-    auto k_step = [&](auto PP, int kt) __attribute__((always_inline)) {
+    // the MFMAs of one K-step from register set P
+    auto mfma_step = [&](auto PP, int kt) __attribute__((always_inline)) {
         constexpr int P = decltype(PP)::value;
-        if(kt + KSTRIDE < KT)
-            load_step(std::integral_constant<int, 1 - P>{}, kt + KSTRIDE);
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
         {
             // scale byte of (K-step parity, 16-row half): tests/contrib/moe/test_fused_moe.py:222-236
             const int kpar = SPLITK ? (kt & 1) : P;          // without the split the parity is the register set
@@ -188,34 +197,70 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
                                                                        acc[j][mt], 0, 0, 0);
         }
     };
-    load_step(std::integral_constant<int, 0>{}, SPLITK ? wave : 0);
-    for(int kt = SPLITK ? wave : 0; kt < KT; kt += 2 * KSTRIDE)
+    const int kt0 = SPLITK ? wave : 0;
+    if constexpr(DEEP)
     {
-        k_step(std::integral_constant<int, 0>{}, kt);
-        if(kt + KSTRIDE < KT)                                          // a wave's share of K-steps may be odd
-            k_step(std::integral_constant<int, 1>{}, kt + KSTRIDE);
+        // ring of three: a register set is refilled, three K-steps of this wave ahead, as soon as its MFMAs are issued
+        using B0 = std::integral_constant<int, 0>;
+        using B1 = std::integral_constant<int, 1>;
+        using B2 = std::integral_constant<int, 2>;
+        load_step(B0{}, kt0);
+        if(kt0 + KSTRIDE < KT)
+            load_step(B1{}, kt0 + KSTRIDE);
+        if(kt0 + 2 * KSTRIDE < KT)
+            load_step(B2{}, kt0 + 2 * KSTRIDE);
+        auto ring_step = [&](auto BB, int kt) __attribute__((always_inline)) {
+            mfma_step(BB, kt);
+            if(kt + 3 * KSTRIDE < KT)
+                load_step(BB, kt + 3 * KSTRIDE);
+        };
+        for(int kt = kt0; kt < KT; kt += 3 * KSTRIDE)
+        {
+            ring_step(B0{}, kt);
+            if(kt + KSTRIDE < KT)
+                ring_step(B1{}, kt + KSTRIDE);
+            if(kt + 2 * KSTRIDE < KT)
+                ring_step(B2{}, kt + 2 * KSTRIDE);
+        }
+    }
+    else
+    {
+        // one K-step from register set P while the next one loads into set 1 - P (K / 128 is even)
+        auto k_step = [&](auto PP, int kt) __attribute__((always_inline)) {
+            constexpr int P = decltype(PP)::value;
+            if(kt + KSTRIDE < KT)
+                load_step(std::integral_constant<int, 1 - P>{}, kt + KSTRIDE);
+            mfma_step(PP, kt);
+        };
+        load_step(std::integral_constant<int, 0>{}, kt0);
+        for(int kt = kt0; kt < KT; kt += 2 * KSTRIDE)
+        {
+            k_step(std::integral_constant<int, 0>{}, kt);
+            if(kt + KSTRIDE < KT)                                          // a wave's share of K-steps may be odd
+                k_step(std::integral_constant<int, 1>{}, kt + KSTRIDE);
+        }
     }
     // which row groups this wave finishes: all four of its own, or (split K) the w-th of the shared ones
     // (stage 1: gate group w and its up group w + 2, waves 0 and 1 only)
     if(SPLITK)
     {
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
 #pragma unroll
             for(int mt = 0; mt < MT; mt++)
-                *(v4f*)&red[(((wave * 4 + j) * MT + mt) * WAVE + lane) * 4] = acc[j][mt];
+                *(v4f*)&red[(((wave * RG + j) * MT + mt) * WAVE + lane) * 4] = acc[j][mt];
         __syncthreads();
-        if(wave >= (STAGE == 1 ? 2 : 4))
+        if(wave >= (STAGE == 1 ? 2 : RG))
             return;
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
 #pragma unroll
             for(int mt = 0; mt < MT; mt++)
             {
                 v4f sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for(int w = 0; w < SPLIT; w++)
-                    sum += *(const v4f*)&red[(((w * 4 + j) * MT + mt) * WAVE + lane) * 4];
+                for(int w = 0; w < NW; w++)
+                    sum += *(const v4f*)&red[(((w * RG + j) * MT + mt) * WAVE + lane) * 4];
                 acc[j][mt] = sum;
             }
     }
@@ -227,7 +272,7 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     if(g.bias)
     {
 #pragma unroll
-        for(int j = 0; j < 4; j++)
+        for(int j = 0; j < RG; j++)
 #pragma unroll
             for(int i = 0; i < 4; i++)
             {
@@ -243,7 +288,7 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     for(int mt = 0; mt < MT; mt++)
     {
         const int p = m_blk * BM + mt * 16 + r;
-        if(STAGE == 1)
+        if constexpr(STAGE == 1)
         {
 #pragma unroll
             for(int j = 0; j < 2; j++)
@@ -263,7 +308,7 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
             const int tok = (int)(ids[mt] & 0xFFFFFFu), slot = (int)(ids[mt] >> 24);
             const float rw = one_token ? g.token_w[m_blk] : g.sorted_w[p];
 #pragma unroll
-            for(int j = 0; j < 4; j++)
+            for(int j = 0; j < RG; j++)
             {
                 if(!mine(j))
                     continue;
@@ -275,7 +320,8 @@ __global__ void __launch_bounds__(SPLIT == 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     }
 }
 
-// split_k: 0 = decide here, 1 = never, 4 / 16 = always that many waves per 64-row tile
+// split_k: 0 = decide here, 1 = never, 4 / 16 = always that many waves per 64-row tile, 32 = sixteen waves per 32-row
+// tile with three K-steps in flight (down GEMM; the gate_up GEMM takes 16 instead)
 template <int STAGE>
 static int launch_w4a16(W4A16Args g, int block_m, int64_t n_blk, int64_t rows, int experts, int split_k,
                         hipStream_t stream)
@@ -285,22 +331,33 @@ static int launch_w4a16(W4A16Args g, int block_m, int64_t n_blk, int64_t rows, i
     if(experts + rows / block_m < blocks)
         blocks = experts + rows / block_m;
     int split = split_k == 1 ? 0 : split_k;
+    if(STAGE == 1 && split == 32)       // (the 32-row tile exists for the down GEMM: gate_up takes sixteen waves, or four)
+        split = g.K >= 2048 ? 16 : 4;
     if(split_k == 0 && blocks * g.n_tiles < 2048)
         // sixteen waves when the four-way split would still start fewer workgroups than there are CUs and the K loop
         // is long enough to matter (Mixtral shape, one token: the layer 54.0 -> 49.7 us; forced onto the gate_up GEMM as well,
         // which already starts 896 workgroups there, 57.5 us)
-        split = (blocks * g.n_tiles * 4 < 256 && g.K >= 8192 && block_m == 16) ? 16 : 4;
+        // (the down GEMM then takes the sixteen-wave split on 32-row tiles with three K-steps in flight, split 32:
+        // Mixtral shape, one token, the down GEMM 16.9 -> see the measurements in the kernel's comment)
+        split = (blocks * g.n_tiles * 4 < 256 && g.K >= 8192 && block_m == 16) ? (STAGE == 2 ? 32 : 16) : 4;
     // (sixteen waves of a workgroup share the register file four to a SIMD: 128 registers each, which only the 16-row
     // tile fits into; and every wave needs a K-step of its own)
-    if(split == 16 && (g.K < 2048 || block_m != 16))
+    if(split >= 16 && (g.K < 2048 || block_m != 16))
     {
-        pyhip_set_error("moe_gemm_w4a16: split_k=16 needs K >= 2048 and block_m = 16 (K=%d, block_m=%d)", g.K, block_m);
+        pyhip_set_error("moe_gemm_w4a16: split_k=16 / 32 need K >= 2048 and block_m = 16 (K=%d, block_m=%d)", g.K, block_m);
         return PYHIP_ERR_INVALID;
     }
     if(split)
-        g.n_tiles *= 4;
+        g.n_tiles *= split == 32 ? 8 : 4;
     // blocks past the bound cannot hold rows (the sort fills blocks from 0 upwards): no workgroups for them
-    dim3 grid((unsigned)(blocks * g.n_tiles)), block(split == 16 ? 1024 : W4A16_THREADS);
+    dim3 grid((unsigned)(blocks * g.n_tiles)), block(split >= 16 ? 1024 : W4A16_THREADS);
+    if constexpr(STAGE == 2)
+        if(split == 32)
+        {
+            hipLaunchKernelGGL((moe_gemm_w4a16_kernel<2, 1, 32>), grid, block, 0, stream, g);
+            PYHIP_CHECK_LAUNCH("moe_gemm_w4a16_kernel");
+            return PYHIP_OK;
+        }
 #define W4A16_CASE(BMV, MTV, SPV) \
     case BMV * 32 + SPV: hipLaunchKernelGGL((moe_gemm_w4a16_kernel<STAGE, MTV, SPV>), grid, block, 0, stream, g); break;
     switch(block_m * 32 + split)
@@ -336,7 +393,7 @@ extern "C" int pyhip_moe_gemm1_w4a16(const void* hidden_bf16, const uint8_t* w1,
                                      int64_t n_blk, int split_k, int activation, float swiglu_limit,
                                      hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm1_w4a16: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16 || split_k == 32, "moe_gemm1_w4a16: split_k=%d not in {0,1,4,16,32}", split_k);
     PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
                   "moe_gemm1_w4a16: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
     int rc = check_w4a16("moe_gemm1_w4a16", hidden_bf16, w1, w1_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
@@ -368,7 +425,7 @@ extern "C" int pyhip_moe_gemm1_w4a16_token(const void* hidden_bf16, const uint8_
                                            int hidden, int inter, int split_k, int activation, float swiglu_limit,
                                            hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm1_w4a16_token: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16 || split_k == 32, "moe_gemm1_w4a16_token: split_k=%d not in {0,1,4,16,32}", split_k);
     PYHIP_REQUIRE(activation == 0 || (activation == 1 && swiglu_limit > 0.f),
                   "moe_gemm1_w4a16_token: activation=%d (0 SiLU, 1 SwiGLU with a positive limit)", activation);
     PYHIP_REQUIRE(hidden_bf16 && w1 && w1_scale && topk_ids && a2_bf16, "moe_gemm1_w4a16_token: null pointer");
@@ -393,7 +450,7 @@ extern "C" int pyhip_moe_gemm2_w4a16_token(const void* a2_bf16, const uint8_t* w
                                            const int32_t* expert_mask, const int32_t* num_local_tokens, void* out3_bf16,
                                            int topk, int experts, int hidden, int inter, int split_k, hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm2_w4a16_token: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16 || split_k == 32, "moe_gemm2_w4a16_token: split_k=%d not in {0,1,4,16,32}", split_k);
     PYHIP_REQUIRE(a2_bf16 && w2 && w2_scale && topk_ids && topk_weights && out3_bf16, "moe_gemm2_w4a16_token: null pointer");
     PYHIP_REQUIRE(inter > 0 && inter % 512 == 0 && hidden > 0 && hidden % 256 == 0,
                   "moe_gemm2_w4a16_token: inter=%d must be a multiple of 512, hidden=%d of 256", inter, hidden);
@@ -418,7 +475,7 @@ extern "C" int pyhip_moe_gemm2_w4a16(const void* a2_bf16, const uint8_t* w2, con
                                      int tokens, int topk, int experts, int hidden, int inter, int block_m,
                                      int64_t n_blk, int split_k, hipStream_t stream)
 {
-    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16, "moe_gemm2_w4a16: split_k=%d not in {0,1,4,16}", split_k);
+    PYHIP_REQUIRE(split_k == 0 || split_k == 1 || split_k == 4 || split_k == 16 || split_k == 32, "moe_gemm2_w4a16: split_k=%d not in {0,1,4,16,32}", split_k);
     int rc = check_w4a16("moe_gemm2_w4a16", a2_bf16, w2, w2_scale, sorted_ids, sorted_expert_ids, num_valid_ids,
                          out3_bf16, inter, block_m, n_blk, hidden / 256);
     if(rc)

@@ -172,7 +172,8 @@ def fused_moe(
     _require(quant_type == QuantType.per_1x32, "this operator is the MXFP4 (per_1x32) path")
     _require(not doweight_stage1, "doweight_stage1 is not supported (the reference rejects it as well)")
     _require(a1_scale is None and a2_scale is None, "activations are quantised dynamically: a1_scale / a2_scale must be None")
-    _require(splitk in (0, 1, 4, 16), "splitk: 0 = automatic, 1 = off, 4 / 16 = split K over that many waves of a workgroup (w4a16 path only)")
+    _require(splitk in (0, 1, 4, 16, 32), "splitk: 0 = automatic, 1 = off, 4 / 16 = split K over that many waves of a workgroup, "
+             "32 = sixteen waves on 32-row weight tiles in the down GEMM (w4a16 path only)")
     _require(w1_scale is not None and w2_scale is not None, "w1_scale and w2_scale (e8m0, shuffled) are required")
     _require(hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and hidden_states.dim() == 2,
              "hidden_states must be a bf16 matrix on the GPU", TypeError)

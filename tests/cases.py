@@ -21,6 +21,9 @@ CONFIGS = {
     # long K in both GEMMs (16 and 20 K-steps of 128): the sixteen-wave split of the bf16-activation kernels, with one
     # K-step per wave in gate_up and an uneven share (one or two) in down
     "longk_s": dict(E=4, k=2, H=2048, I=2560, router="softmax"),
+    # a down GEMM with 68 K-steps: the sixteen-wave split on 32-row tiles gives a wave four or five of them, more than the
+    # three it keeps in flight, and with two experts and four 256-row tiles it is what the launcher picks by itself
+    "verylongk_s": dict(E=2, k=2, H=1024, I=8704, router="softmax"),
 }
 
 

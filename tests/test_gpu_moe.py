@@ -330,6 +330,8 @@ def test_padded_weight_rows_are_not_read(T, bm):
     ("gptoss_s1", 20, 16, True, 4),
     ("odd", 9, 16, False, 0), ("odd", 77, 32, True, 1),
     ("longk_s", 3, 16, True, 16), ("longk_s", 40, 16, False, 16), ("longk_s", 3, 16, False, 4),
+    ("longk_s", 3, 16, True, 32), ("longk_s", 40, 16, False, 32), ("verylongk_s", 2, 16, True, 32), ("verylongk_s", 1, 16, False, 0),
+    ("verylongk_s", 20, 16, True, 0),
 ])
 def test_w4a16_matches_oracle(name, T, bm, bias, splitk):
     """bf16 activations x MXFP4 weights (method="w4a16") against the oracle's "a16" path:
@@ -542,7 +544,7 @@ def test_expert_mask_and_local_tokens(method, T):
 
 
 @pytest.mark.parametrize("name,bias,swiglu", [("mixtral_s", False, False), ("dsv3_s", True, False), ("tiny", True, True),
-                                              ("longk_s", False, False)])
+                                              ("longk_s", False, False), ("verylongk_s", True, False)])
 def test_single_token_skips_the_sort(name, bias, swiglu):
     """One token with bf16 activations: the layer call runs no sort, the GEMMs read topk_ids / topk_weights themselves
     (pyhip_moe_gemm{1,2}_w4a16_token).  The result must equal the sorted, step-by-step path bit for bit (which the
