@@ -77,7 +77,10 @@ __global__ void __launch_bounds__(SPLIT >= 16 ? 1024 : W4A16_THREADS) moe_gemm_w
     constexpr bool DEEP   = SPLIT == 32;
     constexpr int NW      = DEEP ? 16 : SPLIT;    // waves that split K
     constexpr int RG      = DEEP ? 2 : 4;         // 16-row weight row groups of a wave
-    constexpr int NB      = DEEP ? 3 : 2;         // K-steps of operands in registers
+    // K-steps of operands in registers: three where a wave's K loop is a chain of a few memory latencies (the 16-row
+    // tile under a K split; 151-153 registers, three waves per SIMD instead of four: Mixtral shape, 1 / 4 tokens - 3 %,
+    // nothing lost elsewhere), two otherwise
+    constexpr int NB      = (DEEP || (SPLIT == 4 && MT == 1)) ? 3 : 2;
     static_assert(!DEEP || STAGE == 2, "the 32-row tile exists for the down GEMM");
     __shared__ float red[SPLITK ? NW * RG * MT * WAVE * 4 : 1];  // [wave][j][mt][lane][4]
     const int tid = threadIdx.x, lane = tid % WAVE;
@@ -198,7 +201,7 @@ __global__ void __launch_bounds__(SPLIT >= 16 ? 1024 : W4A16_THREADS) moe_gemm_w
         }
     };
     const int kt0 = SPLITK ? wave : 0;
-    if constexpr(DEEP)
+    if constexpr(NB == 3)
     {
         // ring of three: a register set is refilled, three K-steps of this wave ahead, as soon as its MFMAs are issued
         using B0 = std::integral_constant<int, 0>;
