@@ -466,7 +466,7 @@ def test_auto_dispatch():
     assert torch.equal(auto, fused_moe(L.hidden.cuda(), w1, w2, tw, ti, method="a4w4", **kw))
 
 
-@pytest.mark.parametrize("name,T,method", [("dsv3_s", 16, "w4a16"), ("tiny", 300, "a4w4")])
+@pytest.mark.parametrize("name,T,method", [("dsv3_s", 16, "w4a16"), ("tiny", 300, "a4w4"), ("dsv3_s", 1, "w4a16")])
 def test_graph_capture_replays(name, T, method):
     """The whole layer is enqueue-only (no host synchronisation, no memset nodes), so it can be captured in a
     HIP graph; every replay, with the inputs rewritten in place and eager work in between, must reproduce the
@@ -490,7 +490,8 @@ def test_graph_capture_replays(name, T, method):
     for rep in range(3):
         hidden.copy_((torch.randn(T, L.H, generator=g)).to(torch.bfloat16))
         perm = torch.randperm(T, generator=g)
-        ti.copy_(torch.from_numpy(L.topk_ids)[perm])    # a different routing on every replay
+        # a different routing on every replay (one token: its experts shifted, which keeps them distinct)
+        ti.copy_((torch.from_numpy(L.topk_ids)[perm] + (3 * (rep + 1) if T == 1 else 0)) % L.E)
         tw.copy_(torch.from_numpy(L.topk_w)[perm])
         graph.replay()
         torch.cuda.synchronize()
